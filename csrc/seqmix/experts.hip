@@ -1,10 +1,12 @@
 // Mixture of experts: the router with a group-limited choice, the expert matrix products over
 // the routed rows, and the weighted sum of the chosen experts' outputs.
 //
-// group_route_k: z = h . Wr^T in fp32, s = sigmoid(z).  The E experts are cut into `groups`
-// contiguous blocks of equal size; a block is ranked by its top-2 sum of s; experts outside the
-// `keep` best blocks are struck out, and the `top` largest remaining s win (ties: the lower
-// index).  The weights are the winners' s without rescaling.  A token r routed to its k-th expert is slot
+// group_route_k: z = h . Wr^T in fp32, s = sigmoid(z) or softmax(z) over all experts; the
+// choice is made on s plus an optional per-expert correction.  The E experts are cut into
+// `groups` contiguous blocks of equal size; a block is ranked by the sum of its two best choice
+// scores or by its best one; experts outside the `keep` best blocks are struck out, and the
+// `top` largest remaining choice scores win (ties: the lower index).  The weights are the
+// winners' s (without the correction), not rescaled.  A token r routed to its k-th expert is slot
 // r * top + k; every expert gets the list of its slots (cnt / rows).
 //
 // expert_gemm: for expert e and each of its slots s: out[s] = x[s / x_div] . W_e^T.  Rows are
@@ -37,15 +39,20 @@ __device__ __forceinline__ void wave_sync() {
   __builtin_amdgcn_wave_barrier();
 }
 
+// score: 0 sigmoid, 1 softmax over all experts.  corr (optional, [E]): added to the scores for
+// the choice only.  gscore: a group is ranked by 0 the sum of its two best choice scores, 1 its
+// best choice score.
 template <typename T>
 __global__ void __launch_bounds__(256)
 group_route_k(const T* __restrict__ h, int ldh, const float* __restrict__ wr, int W, int E, int top,
-              int groups, int keep, int* __restrict__ ids, float* __restrict__ wts,
-              int* __restrict__ cnt, int* __restrict__ rows, int ldr) {
+              int groups, int keep, int score, const float* __restrict__ corr, int gscore,
+              int* __restrict__ ids, float* __restrict__ wts, int* __restrict__ cnt,
+              int* __restrict__ rows, int ldr) {
   extern __shared__ float smem[];
   float* sh = smem;          // [W] the row in fp32
-  float* ss = sh + W;        // [E] scores; -1 marks "cannot be chosen (any more)"
-  float* sgs = ss + E;       // [groups] group scores
+  float* ss = sh + W;        // [E] scores (the weights of the chosen)
+  float* sc = ss + E;        // [E] choice scores; -inf marks "cannot be chosen (any more)"
+  float* sgs = sc + E;       // [groups] group scores
   const int r = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
   for (int i = threadIdx.x; i < W; i += blockDim.x) sh[i] = ldf(h, (size_t)r * ldh + i);
   __syncthreads();
@@ -69,24 +76,40 @@ group_route_k(const T* __restrict__ h, int ldh, const float* __restrict__ wr, in
     d2 = wave_sum(d2);
     d3 = wave_sum(d3);
     if (lane == 0) {
-      ss[e0] = sigmoidf_(d0);
-      if (e0 + 1 < E) ss[e0 + 1] = sigmoidf_(d1);
-      if (e0 + 2 < E) ss[e0 + 2] = sigmoidf_(d2);
-      if (e0 + 3 < E) ss[e0 + 3] = sigmoidf_(d3);
+      ss[e0] = score ? d0 : sigmoidf_(d0);
+      if (e0 + 1 < E) ss[e0 + 1] = score ? d1 : sigmoidf_(d1);
+      if (e0 + 2 < E) ss[e0 + 2] = score ? d2 : sigmoidf_(d2);
+      if (e0 + 3 < E) ss[e0 + 3] = score ? d3 : sigmoidf_(d3);
     }
   }
   __syncthreads();
   if (wave != 0) return;
+  if (score) {   // softmax over all experts
+    float mx = -INFINITY;
+    for (int e = lane; e < E; e += 64) mx = fmaxf(mx, ss[e]);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+    float sum = 0.0f;
+    for (int e = lane; e < E; e += 64) {
+      float v = expf(ss[e] - mx);
+      ss[e] = v;
+      sum += v;
+    }
+    sum = wave_sum(sum);
+    for (int e = lane; e < E; e += 64) ss[e] = ss[e] / sum;
+  }
+  for (int e = lane; e < E; e += 64) sc[e] = corr ? ss[e] + corr[e] : ss[e];
+  wave_sync();
   const int per = E / groups;
   if (keep < groups) {
     for (int g = lane; g < groups; g += 64) {
-      float b1 = -1.0f, b2 = -1.0f;   // top-2 of the block
+      float b1 = -INFINITY, b2 = -INFINITY;   // top-2 of the block
       for (int i = 0; i < per; i++) {
-        float v = ss[g * per + i];
+        float v = sc[g * per + i];
         if (v > b1) { b2 = b1; b1 = v; }
         else if (v > b2) b2 = v;
       }
-      sgs[g] = b1 + (per > 1 ? b2 : 0.0f);
+      sgs[g] = b1 + ((per > 1 && gscore == 0) ? b2 : 0.0f);
     }
     wave_sync();
     // keep the best groups: pick `keep` times, then strike out the experts of the others
@@ -102,22 +125,22 @@ group_route_k(const T* __restrict__ h, int ldh, const float* __restrict__ wr, in
       wave_sync();
     }
     for (int e = lane; e < E; e += 64)
-      if (sgs[e / per] != -INFINITY) ss[e] = -1.0f;
+      if (sgs[e / per] != -INFINITY) sc[e] = -INFINITY;
     wave_sync();
   }
   for (int k = 0; k < top; k++) {
     float bv = -INFINITY;
     int bi = 1 << 30;
     for (int e = lane; e < E; e += 64) {
-      float v = ss[e];
+      float v = sc[e];
       if (v > bv) { bv = v; bi = e; }
     }
     wave_argmax(bv, bi);
     if (lane == 0) {
-      ss[bi] = -2.0f;
+      sc[bi] = -INFINITY;
       int slot = r * top + k;
       ids[slot] = bi;
-      wts[slot] = bv;
+      wts[slot] = ss[bi];
       int at = atomicAdd(&cnt[bi], 1);
       rows[(size_t)bi * ldr + at] = slot;
     }
@@ -188,6 +211,15 @@ __device__ __forceinline__ float expert_act(float g, float u, float limit, float
   return g * sigmoidf_(alpha * g) * (u + 1.0f);
 }
 
+// epi = 2: an ungated unit, every product passes relu(.)^2; epi = 0: the products themselves
+__device__ __forceinline__ float plain_epi(float v, int epi) {
+  if (epi == 2) {
+    v = fmaxf(v, 0.0f);
+    v *= v;
+  }
+  return v;
+}
+
 // bf16 on the matrix cores, few slots per expert (decode-sized steps): a block takes 16 slots x
 // 64 output columns of one expert and its four wavefronts split K among themselves, so the
 // chain of dependent loads is a quarter as long; each wavefront walks its share in steps of 32
@@ -256,7 +288,7 @@ expert_gemm_mfma_k(const bf16* __restrict__ x, int ldx, int x_div, const bf16* _
   for (int i = 0; i < 4; i++) {
     int so = __shfl(slot, quad * 4 + i, 64);
     if (so < 0) continue;
-    if (epi) {
+    if (epi == 1) {
 #pragma unroll
       for (int t = 0; t < 4; t += 2) {
         int n = n0 + t * 16;
@@ -269,7 +301,7 @@ expert_gemm_mfma_k(const bf16* __restrict__ x, int ldx, int x_div, const bf16* _
 #pragma unroll
     for (int t = 0; t < 4; t++) {
       int n = n0 + t * 16 + n16;
-      if (n < N) out[(size_t)so * ldo + n] = __float2bfloat16(acc[t][i]);
+      if (n < N) out[(size_t)so * ldo + n] = __float2bfloat16(plain_epi(acc[t][i], epi));
     }
   }
 }
@@ -364,7 +396,7 @@ expert_gemm_mfma_big_k(const bf16* __restrict__ x, int ldx, int x_div, const bf1
     for (int i = 0; i < 4; i++) {
       int so = sslot[wm + a * 16 + quad * 4 + i];
       if (so < 0) continue;
-      if (epi) {
+      if (epi == 1) {
 #pragma unroll
         for (int b = 0; b < 4; b += 2) {
           int n = n0 + wn + b * 16;
@@ -377,7 +409,7 @@ expert_gemm_mfma_big_k(const bf16* __restrict__ x, int ldx, int x_div, const bf1
 #pragma unroll
       for (int b = 0; b < 4; b++) {
         int n = n0 + wn + b * 16 + n16;
-        if (n < N) out[(size_t)so * ldo + n] = __float2bfloat16(acc[a][b][i]);
+        if (n < N) out[(size_t)so * ldo + n] = __float2bfloat16(plain_epi(acc[a][b][i], epi));
       }
     }
   }
@@ -433,7 +465,7 @@ expert_gemm_fma_k(const T* __restrict__ x, int ldx, int x_div, const T* __restri
   for (int a = 0; a < 2; a++) {
     int s = sslot[ty * 2 + a];
     if (s < 0) continue;
-    if (epi) {
+    if (epi == 1) {
 #pragma unroll
       for (int u = 0; u < 4; u += 2) {
         int n = n0 + 16 * u;
@@ -445,18 +477,26 @@ expert_gemm_fma_k(const T* __restrict__ x, int ldx, int x_div, const T* __restri
 #pragma unroll
     for (int u = 0; u < 4; u++) {
       int n = n0 + tx + 16 * u;
-      if (n < N) stf(out, (size_t)s * ldo + n, acc[a][u]);
+      if (n < N) stf(out, (size_t)s * ldo + n, plain_epi(acc[a][u], epi));
     }
   }
 }
 
+// out[r] = sum_k wts[r, k] * y[r * top + k]; a slot whose expert index is >= n_real (ids given)
+// stands for an expert that hands its input back: its term is wts * x[r]
 template <typename T>
 __global__ void expert_combine_k(const T* __restrict__ y, int ldy, const float* __restrict__ wts,
-                                 T* __restrict__ out, int ldo, int top, int n) {
+                                 T* __restrict__ out, int ldo, int top, int n,
+                                 const int* __restrict__ ids, int n_real, const T* __restrict__ x,
+                                 int ldx) {
   int c = blockIdx.x * blockDim.x + threadIdx.x, r = blockIdx.y;
   if (c >= n) return;
   float s = 0.0f;
-  for (int k = 0; k < top; k++) s += wts[r * top + k] * ldf(y, (size_t)(r * top + k) * ldy + c);
+  for (int k = 0; k < top; k++) {
+    bool same = ids && ids[r * top + k] >= n_real;
+    float v = same ? ldf(x, (size_t)r * ldx + c) : ldf(y, (size_t)(r * top + k) * ldy + c);
+    s += wts[r * top + k] * v;
+  }
   stf(out, (size_t)r * ldo + c, s);
 }
 
@@ -464,17 +504,17 @@ extern "C" {
 
 // cnt must be zero on entry
 int p2p_sm_group_route(const void* h, int ldh, const float* wr, int R, int W, int E, int top,
-                       int groups, int keep, int* ids, float* wts, int* cnt, int* rows, int ldr,
-                       int f32, hipStream_t st) {
+                       int groups, int keep, int score, const float* corr, int gscore, int* ids,
+                       float* wts, int* cnt, int* rows, int ldr, int f32, hipStream_t st) {
   if (R <= 0) return 0;
   if (E < 1 || groups < 1 || E % groups || keep < 1 || keep > groups || top < 1 ||
       top > keep * (E / groups) || ldr < R * top)
     return (int)hipErrorInvalidValue;
-  size_t shm = (size_t)(W + E + groups) * 4;
+  size_t shm = (size_t)(W + 2 * E + groups) * 4;
   if (shm > 64 * 1024) return (int)hipErrorInvalidValue;
   SM_DISPATCH_T(f32, hipLaunchKernelGGL(group_route_k<T>, dim3(R), dim3(256), shm, st,
-                                         (const T*)h, ldh, wr, W, E, top, groups, keep, ids, wts,
-                                         cnt, rows, ldr));
+                                         (const T*)h, ldh, wr, W, E, top, groups, keep, score, corr,
+                                         gscore, ids, wts, cnt, rows, ldr));
   return (int)hipGetLastError();
 }
 
@@ -486,7 +526,7 @@ int p2p_sm_expert_gemm(const void* x, int ldx, int x_div, const void* w, const i
                        int total_slots, int epi, float limit, float alpha, int f32,
                        hipStream_t st) {
   if (total_slots <= 0 || E <= 0) return 0;
-  if (x_div < 1 || N < 1 || K < 1 || (epi && N % 32)) return (int)hipErrorInvalidValue;
+  if (x_div < 1 || N < 1 || K < 1 || (epi == 1 && N % 32)) return (int)hipErrorInvalidValue;
   if (!f32 && K % 8 == 0 && ldx % 8 == 0 && ((size_t)x & 15) == 0 && ((size_t)w & 15) == 0) {
     if (total_slots >= 64 * E) {   // prompts: the large tile
       int tmp = (((total_slots + 127) / 128 + E) + 7) & ~7;
@@ -510,11 +550,13 @@ int p2p_sm_expert_gemm(const void* x, int ldx, int x_div, const void* w, const i
 }
 
 int p2p_sm_expert_combine(const void* y, int ldy, const float* wts, void* out, int ldo, int R,
-                          int top, int n, int f32, hipStream_t st) {
+                          int top, int n, const int* ids, int n_real, const void* x, int ldx,
+                          int f32, hipStream_t st) {
   if (R <= 0) return 0;
+  if (ids && !x) return (int)hipErrorInvalidValue;
   dim3 g((n + 255) / 256, R), b(256);
   SM_DISPATCH_T(f32, hipLaunchKernelGGL(expert_combine_k<T>, g, b, 0, st, (const T*)y, ldy, wts,
-                                         (T*)out, ldo, top, n));
+                                         (T*)out, ldo, top, n, ids, n_real, (const T*)x, ldx));
   return (int)hipGetLastError();
 }
 

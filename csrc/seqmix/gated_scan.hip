@@ -7,6 +7,16 @@
 // followed by the head's RMS norm over V, a weight shared by the heads and, for the delta
 // rule, a sigmoid output gate.
 //
+// The matrix memory of the mLSTM is the plain write with a scalar decay per head and a
+// normaliser: with log gates i_t, f_t and the running maximum m_t = max(f_t + m_(t-1), i_t)
+// (m_0 = 0),  a_t = exp(f_t + m_(t-1) - m_t),  b_t = exp(i_t - m_t),
+//   S <- a_t S + (b_t k) v^T,  n <- a_t n + b_t k,  o = S^T q / (max(|n . q|, exp(-m_t)) + 1e-6).
+// m_t depends on the gates alone, so a small kernel walks it first (mlstm_gates_k: a_t, b_t and
+// exp(-m_t) per token and head, the slot keeps m); with these coefficients the recurrence is
+// linear in (S, n) and runs here -- n is one more value column of the state, written with the
+// value 1, so n . q leaves the kernel as column V of S^T q.  The head's o is RMS-normalised,
+// weighted per channel of the head and gated by a sigmoid.
+//
 // The value columns of S are independent.  A wavefront covers 16 columns x 4 slices of the key
 // index; lane (c, s) keeps rows s*DQ .. s*DQ+DQ-1 of column c in registers (NC columns, 16
 // apart, in the general form of the kernel), and the sums over the key index (S^T k before
@@ -38,6 +48,10 @@ struct ScanArgs {
   const void* braw; int ldb;
   const void* gate; int ldg;
   const float* A_log; const float* dt_bias;
+  // matrix memory: proj = [q (H*D) | k (H*D) | v (H*V) | gate (H*V) | ...] and the
+  // coefficients (a_t, b_t, exp(-m_t)) fp32 [rows, H, 3]
+  const float* coef;
+  int VS;   // value columns of the state: V, or V + 1 with the normaliser
   // common
   const float* normw; float* state; const int* ent; void* out; int ldo;
   int H, G, D, V, CT;
@@ -52,16 +66,17 @@ struct ScanArgs {
   float* chunk_trans;   // [chunks, H, D, D]
 };
 
-template <typename T, int DQ, bool DELTA, int NC>
+template <typename T, int DQ, int KIND, int NC>   // KIND 0: plain write (HGRN2), 1: delta rule, 2: matrix memory
 __global__ void __launch_bounds__(1024 / NC) gated_scan_k(ScanArgs a) {
+  constexpr bool DELTA = KIND == 1, MEM = KIND == 2;
   constexpr int DKP = 4 * DQ;   // padded key index (zero filled in LDS)
   constexpr int WC = 16 * NC;   // columns per wavefront: a lane keeps NC columns, 16 apart
-  const int H = a.H, D = a.D, V = a.V, CT = a.CT, mode = a.mode;
+  const int H = a.H, D = a.D, V = a.V, VS = a.VS, CT = a.CT, mode = a.mode;
   const int e = blockIdx.x / H, h = blockIdx.x % H;
   const Entry en = load_entry(a.ent, e);
   if (en.n <= 0) return;
   const bool trans = mode == 3;
-  const int NCOL = trans ? D : V;              // columns of the matrix this block carries
+  const int NCOL = trans ? D : VS;             // columns of the matrix this block carries
   const int nw = blockDim.x >> 6, VP = nw * WC;
   extern __shared__ __align__(16) float smem[];
   float* sq = smem;                  // [CT][DKP]
@@ -88,9 +103,9 @@ __global__ void __launch_bounds__(1024 / NC) gated_scan_k(ScanArgs a) {
   const T* gate = (const T*)a.gate;
   T* out = (T*)a.out;
   float S[NC][DQ];
-  float* Sg = mode == 0 ? a.state + ((size_t)en.slot * H + h) * D * V
+  float* Sg = mode == 0 ? a.state + ((size_t)en.slot * H + h) * D * VS
             : trans     ? a.chunk_trans + ((size_t)en.slot * H + h) * D * D
-                        : a.chunk_state + ((size_t)en.slot * H + h) * D * V;
+                        : a.chunk_state + ((size_t)en.slot * H + h) * D * VS;
   const bool from_state = mode == 2 || (mode == 0 && en.start > 0);
 #pragma unroll
   for (int c = 0; c < NC; c++)
@@ -104,7 +119,7 @@ __global__ void __launch_bounds__(1024 / NC) gated_scan_k(ScanArgs a) {
   if (!DELTA && mode == 1)
     for (int i = threadIdx.x; i < DKP; i += blockDim.x) sP[i] = 1.0f;
   const float negA = DELTA ? -expf(a.A_log[h]) : 0.0f;
-  const float qscale = DELTA ? 1.0f / sqrtf((float)D) : 1.0f;
+  const float qscale = (DELTA || MEM) ? 1.0f / sqrtf((float)D) : 1.0f;
   for (int t0 = 0; t0 < en.n; t0 += CT) {
     const int ct = min(CT, en.n - t0);
     for (int idx = threadIdx.x; idx < ct * DKP; idx += blockDim.x) {
@@ -117,6 +132,11 @@ __global__ void __launch_bounds__(1024 / NC) gated_scan_k(ScanArgs a) {
           vk = a.conv[row * a.ldc + a.G * D + hk * D + i];
           float dt = softplusf_(ldf(araw, row * a.lda + h * D + i) + a.dt_bias[h * D + i]);
           vg = expf(negA * dt);
+        } else if (MEM) {
+          const float* cf = a.coef + (row * H + h) * 3;
+          vq = ldf(proj, row * a.ldp + h * D + i) * qscale;
+          vk = cf[1] * ldf(proj, row * a.ldp + H * D + h * D + i);
+          vg = cf[0];
         } else {
           float qr = ldf(proj, row * a.ldp + h * D + i);
           vq = qr * sigmoidf_(qr);
@@ -134,6 +154,7 @@ __global__ void __launch_bounds__(1024 / NC) gated_scan_k(ScanArgs a) {
         float vv = 0.0f;
         if (i < V) vv = DELTA ? a.conv[row * a.ldc + 2 * a.G * D + h * V + i]
                               : ldf(proj, row * a.ldp + 2 * H * D + h * V + i);
+        else if (MEM && i == V) vv = 1.0f;   // the normaliser's column
         sv[idx] = vv;
       }
     if (DELTA) {
@@ -229,14 +250,25 @@ __global__ void __launch_bounds__(1024 / NC) gated_scan_k(ScanArgs a) {
     __syncthreads();
     if (mode == 0 || mode == 2)
     for (int t = wave; t < ct; t += nw) {
+      size_t row = (size_t)(en.row0 + t0 + t);
+      float den = 1.0f;
+      if (MEM) den = fmaxf(fabsf(so[t * VP + V]), a.coef[(row * H + h) * 3 + 2]) + 1e-6f;
       float ss = 0.0f;
-      for (int i = lane; i < V; i += 64) ss += so[t * VP + i] * so[t * VP + i];
+      for (int i = lane; i < V; i += 64) {
+        float o = MEM ? so[t * VP + i] / den : so[t * VP + i];
+        ss += o * o;
+      }
       ss = wave_sum(ss);
       float rs = a.out_scale / sqrtf(ss / (float)V + a.eps);
-      size_t row = (size_t)(en.row0 + t0 + t);
       for (int i = lane; i < V; i += 64) {
-        float y = so[t * VP + i] * rs * a.normw[i];
-        if (DELTA) y *= sigmoidf_(ldf(gate, row * a.ldg + h * V + i));
+        float y;
+        if (MEM) {
+          y = so[t * VP + i] / den * rs * a.normw[h * V + i];
+          y *= sigmoidf_(ldf(proj, row * a.ldp + 2 * H * D + H * V + h * V + i));
+        } else {
+          y = so[t * VP + i] * rs * a.normw[i];
+          if (DELTA) y *= sigmoidf_(ldf(gate, row * a.ldg + h * V + i));
+        }
         stf(out, row * a.ldo + h * V + i, y);
       }
     }
@@ -336,12 +368,64 @@ dense_chain_k(float* __restrict__ cs, const float* __restrict__ trans, float* __
     for (int i = rg; i < D; i += DC_RG) sg[(size_t)i * V + j] = scur[i * LD + col];
 }
 
-template <bool DELTA>
+// Log gates of the matrix memory and their running maximum, one wavefront per (portion, head):
+//   i_t = cap tanh((zi_t + bi) / cap),  f_t = logsigmoid(cap tanh((zf_t + bf) / cap)),
+//   m_t = max(f_t + m_(t-1), i_t)  (m = 0 before position 0; the slot keeps it between steps),
+//   coef[t] = (exp(f_t + m_(t-1) - m_t), exp(i_t - m_t), exp(-m_t)).
+// The gates of 64 tokens are evaluated side by side, lane 0 walks the maximum through them.
+__device__ __forceinline__ float logsigmoidf_(float x) {
+  return fminf(x, 0.0f) - log1pf(expf(-fabsf(x)));
+}
+
+template <typename T>
+__global__ void __launch_bounds__(64)
+mlstm_gates_k(const T* __restrict__ proj, int ldp, int off_i, int off_f,
+              const float* __restrict__ bi, const float* __restrict__ bf, float cap,
+              float* __restrict__ mstate, const int* __restrict__ ent, float* __restrict__ coef,
+              int H) {
+  __shared__ float si[64], sf[64], sm_[65];
+  const int e = blockIdx.x / H, h = blockIdx.x % H, lane = threadIdx.x;
+  const Entry en = load_entry(ent, e);
+  if (en.n <= 0) return;
+  float* mg = mstate + (size_t)en.slot * H + h;
+  float m = en.start > 0 ? *mg : 0.0f;
+  for (int t0 = 0; t0 < en.n; t0 += 64) {
+    const int ct = min(64, en.n - t0);
+    const size_t row = (size_t)(en.row0 + t0 + min(lane, ct - 1));
+    float it = cap * tanhf((ldf(proj, row * ldp + off_i + h) + bi[h]) / cap);
+    float ft = logsigmoidf_(cap * tanhf((ldf(proj, row * ldp + off_f + h) + bf[h]) / cap));
+    si[lane] = it;
+    sf[lane] = ft;
+    __syncthreads();
+    if (lane == 0) {
+      float mm = m;
+      sm_[0] = mm;
+      for (int j = 0; j < ct; j++) {
+        mm = fmaxf(sf[j] + mm, si[j]);
+        sm_[j + 1] = mm;
+      }
+    }
+    __syncthreads();
+    if (lane < ct) {
+      float mp = sm_[lane], mn = sm_[lane + 1];
+      float* cf = coef + (row * H + h) * 3;
+      cf[0] = expf(ft + mp - mn);
+      cf[1] = expf(it - mn);
+      cf[2] = expf(-mn);
+    }
+    m = sm_[ct];
+    __syncthreads();
+  }
+  if (lane == 0) *mg = m;
+}
+
+template <int KIND>
 static int launch_scan(ScanArgs a, int E, int f32, hipStream_t st) {
   if (E <= 0) return 0;
-  if (a.H < 1 || a.D < 1 || a.V < 1 || a.D > 256 || a.V > 256 || a.G < 1 || a.H % a.G)
+  if (KIND != 2) a.VS = a.V;
+  if (a.H < 1 || a.D < 1 || a.V < 1 || a.D > 256 || a.VS > 256 || a.G < 1 || a.H % a.G)
     return (int)hipErrorInvalidValue;
-  int cols = a.mode == 3 ? a.D : a.V;
+  int cols = a.mode == 3 ? a.D : a.VS;
   int dq = a.D <= 32 ? 8 : a.D <= 64 ? 16 : a.D <= 128 ? 32 : 64;
   // one column per lane: two (NC = 2) halve the wavefronts that read the staged vectors from
   // LDS but measured no faster (120 us against 110 us per 64-token pass at 128 x 128 states)
@@ -354,7 +438,7 @@ static int launch_scan(ScanArgs a, int E, int f32, hipStream_t st) {
   size_t shm = (size_t)(CT * per_tok + 4 * dq) * 4;
   dim3 grid(E * a.H), block(64 * nw);
 #define GS(DQ, NC)                                                                            \
-  SM_DISPATCH_T(f32, hipLaunchKernelGGL((gated_scan_k<T, DQ, DELTA, NC>), grid, block, shm, st, a))
+  SM_DISPATCH_T(f32, hipLaunchKernelGGL((gated_scan_k<T, DQ, KIND, NC>), grid, block, shm, st, a))
   if (dq == 8) GS(8, 1);
   else if (dq == 16) GS(16, 1);
   else if (dq == 32) GS(32, 1);
@@ -365,28 +449,30 @@ static int launch_scan(ScanArgs a, int E, int f32, hipStream_t st) {
 
 // the three passes over `NV` chunks (vent) of `E` portions (cent = first chunk, chunks, first
 // position, slot); cs [NV, H, D, V], cd [NV, H, D] (plain write) or ct [NV, H, D, D] (delta rule)
-template <bool DELTA>
+template <int KIND>
 static int launch_chunked(ScanArgs a, const int* vent, int NV, const int* cent, int E, float* cs,
                           float* cd, float* ct, int f32, hipStream_t st) {
+  constexpr bool DELTA = KIND == 1;
   if (NV <= 0 || E <= 0) return 0;
+  if (KIND != 2) a.VS = a.V;
   float* state = a.state;
   a.ent = vent;
   a.chunk_state = cs; a.chunk_decay = cd; a.chunk_trans = ct;
   a.mode = 1;
-  int err = launch_scan<DELTA>(a, NV, f32, st);
+  int err = launch_scan<KIND>(a, NV, f32, st);
   if (err) return err;
   if (DELTA) {
     a.mode = 3;
-    if ((err = launch_scan<DELTA>(a, NV, f32, st))) return err;
+    if ((err = launch_scan<KIND>(a, NV, f32, st))) return err;
     hipLaunchKernelGGL(dense_chain_k, dim3((a.V + DC_COLS - 1) / DC_COLS, E * a.H), dim3(256),
                        (size_t)a.D * (DC_COLS + 1) * 4, st, cs, ct, state, cent, a.H, a.D, a.V);
   } else {
-    hipLaunchKernelGGL(diag_chain_k, dim3((a.D * a.V + 255) / 256, E * a.H), dim3(256), 0, st, cs,
-                       cd, state, cent, a.H, a.D, a.V);
+    hipLaunchKernelGGL(diag_chain_k, dim3((a.D * a.VS + 255) / 256, E * a.H), dim3(256), 0, st, cs,
+                       cd, state, cent, a.H, a.D, a.VS);
   }
   if ((err = (int)hipGetLastError())) return err;
   a.mode = 2;
-  return launch_scan<DELTA>(a, NV, f32, st);
+  return launch_scan<KIND>(a, NV, f32, st);
 }
 
 extern "C" {
@@ -398,7 +484,7 @@ int p2p_sm_hgrn2_scan(const void* proj, int ldp, const float* lower, const float
   a.proj = proj; a.ldp = ldp; a.lower = lower; a.fb = fb;
   a.normw = normw; a.state = state; a.ent = ent; a.out = out; a.ldo = ldo;
   a.H = H; a.G = H; a.D = D; a.V = V; a.eps = eps; a.out_scale = out_scale;
-  return launch_scan<false>(a, E, f32, st);
+  return launch_scan<0>(a, E, f32, st);
 }
 
 int p2p_sm_gated_delta_scan(const float* conv, int ldc, const void* araw, int lda,
@@ -411,7 +497,7 @@ int p2p_sm_gated_delta_scan(const float* conv, int ldc, const void* araw, int ld
   a.gate = gate; a.ldg = ldg; a.A_log = A_log; a.dt_bias = dt_bias;
   a.normw = normw; a.state = state; a.ent = ent; a.out = out; a.ldo = ldo;
   a.H = H; a.G = G; a.D = D; a.V = V; a.eps = eps; a.out_scale = out_scale;
-  return launch_scan<true>(a, E, f32, st);
+  return launch_scan<1>(a, E, f32, st);
 }
 
 int p2p_sm_hgrn2_scan_chunked(const void* proj, int ldp, const float* lower, const float* fb,
@@ -423,7 +509,7 @@ int p2p_sm_hgrn2_scan_chunked(const void* proj, int ldp, const float* lower, con
   a.proj = proj; a.ldp = ldp; a.lower = lower; a.fb = fb;
   a.normw = normw; a.state = state; a.out = out; a.ldo = ldo;
   a.H = H; a.G = H; a.D = D; a.V = V; a.eps = eps; a.out_scale = out_scale;
-  return launch_chunked<false>(a, vent, NV, cent, E, cs, cd, nullptr, f32, st);
+  return launch_chunked<0>(a, vent, NV, cent, E, cs, cd, nullptr, f32, st);
 }
 
 int p2p_sm_gated_delta_scan_chunked(const float* conv, int ldc, const void* araw, int lda,
@@ -438,7 +524,32 @@ int p2p_sm_gated_delta_scan_chunked(const float* conv, int ldc, const void* araw
   a.gate = gate; a.ldg = ldg; a.A_log = A_log; a.dt_bias = dt_bias;
   a.normw = normw; a.state = state; a.out = out; a.ldo = ldo;
   a.H = H; a.G = G; a.D = D; a.V = V; a.eps = eps; a.out_scale = out_scale;
-  return launch_chunked<true>(a, vent, NV, cent, E, cs, nullptr, ct, f32, st);
+  return launch_chunked<1>(a, vent, NV, cent, E, cs, nullptr, ct, f32, st);
+}
+
+// Matrix memory: proj = [q (H*D) | k (H*D) | v (H*V) | gate (H*V) | zi (H) | zf (H)] in the
+// activation type; state fp32 [slots, H, D, V + 1] (column V: the normaliser), mstate fp32
+// [slots, H]; coef fp32 [rows, H, 3] scratch; normw fp32 [H*V].  With NV > 0 the portions run
+// as chunks (vent / cent / cs [NV, H, D, V+1] / cd [NV, H, D]), else in one pass over `ent`.
+int p2p_sm_mlstm_scan(const void* proj, int ldp, const float* bi, const float* bf, float cap,
+                      const float* normw, float* state, float* mstate, float* coef,
+                      const int* ent, int E, float* cs, float* cd, const int* vent, int NV,
+                      const int* cent, void* out, int ldo, int H, int D, int V, float eps,
+                      float out_scale, int f32, hipStream_t st) {
+  if (E <= 0) return 0;
+  if (H < 1 || D < 1 || V < 1 || D > 256 || V > 255 || cap <= 0.0f) return (int)hipErrorInvalidValue;
+  const int off_i = 2 * H * D + 2 * H * V, off_f = off_i + H;
+  SM_DISPATCH_T(f32, hipLaunchKernelGGL(mlstm_gates_k<T>, dim3(E * H), dim3(64), 0, st,
+                                         (const T*)proj, ldp, off_i, off_f, bi, bf, cap, mstate,
+                                         ent, coef, H));
+  int err = (int)hipGetLastError();
+  if (err) return err;
+  ScanArgs a = {};
+  a.proj = proj; a.ldp = ldp; a.coef = coef; a.VS = V + 1;
+  a.normw = normw; a.state = state; a.ent = ent; a.out = out; a.ldo = ldo;
+  a.H = H; a.G = H; a.D = D; a.V = V; a.eps = eps; a.out_scale = out_scale;
+  if (NV > 0) return launch_chunked<2>(a, vent, NV, cent, E, cs, cd, nullptr, f32, st);
+  return launch_scan<2>(a, E, f32, st);
 }
 
 }  // extern "C"

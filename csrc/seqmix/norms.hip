@@ -134,6 +134,56 @@ __global__ void norm_scale_add_k(float* __restrict__ x, const T* __restrict__ y,
     stf(h, (size_t)r * ldh + i, xr[i] * r2 * w2[i]);
 }
 
+// x += a (+ b) on the fp32 residual, the addends summed first (fp32); with w2 also the next
+// layer's input h = x / sqrt(mean(x^2) + eps) * w2 from the updated row
+template <typename T>
+__global__ void add_norm_k(float* __restrict__ x, const T* __restrict__ a, int lda,
+                           const T* __restrict__ b, int ldb, int n, float eps,
+                           const float* __restrict__ w2, T* __restrict__ h, int ldh) {
+  __shared__ float red[16];
+  int r = blockIdx.x;
+  const T* ar = a + (size_t)r * lda;
+  const T* br = b ? b + (size_t)r * ldb : nullptr;
+  float* xr = x + (size_t)r * n;
+  if (n <= NV * (int)blockDim.x) {
+    float xv[NV], wv[NV];
+    float s2 = 0.0f;
+#pragma unroll
+    for (int k = 0; k < NV; k++) {
+      int i = threadIdx.x + k * blockDim.x;
+      bool ok = i < n;
+      float y = ok ? ldf(ar, i) : 0.0f;
+      if (br && ok) y += ldf(br, i);
+      wv[k] = (ok && w2) ? w2[i] : 0.0f;
+      xv[k] = ok ? xr[i] + y : 0.0f;
+      if (ok) xr[i] = xv[k];
+      s2 += xv[k] * xv[k];
+    }
+    if (!w2) return;
+    s2 = block_sum(s2, red);
+    float r2 = 1.0f / sqrtf(s2 / (float)n + eps);
+#pragma unroll
+    for (int k = 0; k < NV; k++) {
+      int i = threadIdx.x + k * blockDim.x;
+      if (i < n) stf(h, (size_t)r * ldh + i, xv[k] * r2 * wv[k]);
+    }
+    return;
+  }
+  float s2 = 0.0f;
+  for (int i = threadIdx.x; i < n; i += blockDim.x) {
+    float y = ldf(ar, i);
+    if (br) y += ldf(br, i);
+    float v = xr[i] + y;
+    xr[i] = v;
+    s2 += v * v;
+  }
+  if (!w2) return;
+  s2 = block_sum(s2, red);
+  float r2 = 1.0f / sqrtf(s2 / (float)n + eps);
+  for (int i = threadIdx.x; i < n; i += blockDim.x)   // each thread re-reads its own writes
+    stf(h, (size_t)r * ldh + i, xr[i] * r2 * w2[i]);
+}
+
 // out[r] = embed[ids[r]] as fp32, and (optionally) the same row in the activation type
 template <typename T>
 __global__ void embed_rows_k(const T* __restrict__ embed, const int* __restrict__ ids,
@@ -259,6 +309,14 @@ int p2p_sm_norm_scale_add(float* x, const void* y, int ldy, const float* w, cons
   if (R <= 0) return 0;
   SM_DISPATCH_T(f32, hipLaunchKernelGGL(norm_scale_add_k<T>, dim3(R), dim3(256), 0, st, x,
                                          (const T*)y, ldy, w, ls, n, eps, w2, (T*)h, ldh));
+  return (int)hipGetLastError();
+}
+
+int p2p_sm_add_norm(float* x, const void* a, int lda, const void* b, int ldb, int R, int n,
+                    float eps, const float* w2, void* h, int ldh, int f32, hipStream_t st) {
+  if (R <= 0) return 0;
+  SM_DISPATCH_T(f32, hipLaunchKernelGGL(add_norm_k<T>, dim3(R), dim3(256), 0, st, x, (const T*)a,
+                                         lda, (const T*)b, ldb, n, eps, w2, (T*)h, ldh));
   return (int)hipGetLastError();
 }
 

@@ -32,12 +32,32 @@ __global__ void ff_act_k(const T* __restrict__ gu, int ld, T* __restrict__ out, 
   stf(out, (size_t)r * ldo + c, g * sigmoidf_(alpha * g) * (u + 1.0f));
 }
 
+// tanh form of gelu: 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))
+__device__ __forceinline__ float gelu_tanhf_(float z) {
+  return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+
+// [gate | up] -> act(gate) * up; act: 0 silu, 1 gelu (tanh form)
 template <typename T>
-__global__ void glu_act_k(const T* __restrict__ gu, int ld, T* __restrict__ out, int ldo, int F) {
+__global__ void glu_act_k(const T* __restrict__ gu, int ld, T* __restrict__ out, int ldo, int F,
+                          int act) {
   int c = blockIdx.x * blockDim.x + threadIdx.x, r = blockIdx.y;
   if (c >= F) return;
   float g = ldf(gu, (size_t)r * ld + c);
-  stf(out, (size_t)r * ldo + c, g * sigmoidf_(g) * ldf(gu, (size_t)r * ld + F + c));
+  float a = act == 1 ? gelu_tanhf_(g) : g * sigmoidf_(g);
+  stf(out, (size_t)r * ldo + c, a * ldf(gu, (size_t)r * ld + F + c));
+}
+
+// out[r, c] = relu(u[r, c])^2 * sigmoid(g[r]): an ungated squared-relu unit whose result is
+// weighted by one gate per row (g == nullptr: no gate)
+template <typename T>
+__global__ void relu2_gate_k(const T* __restrict__ u, int ld, const T* __restrict__ g, int ldg,
+                             T* __restrict__ out, int ldo, int F) {
+  int c = blockIdx.x * blockDim.x + threadIdx.x, r = blockIdx.y;
+  if (c >= F) return;
+  float v = fmaxf(ldf(u, (size_t)r * ld + c), 0.0f);
+  float w = g ? sigmoidf_(ldf(g, (size_t)r * ldg)) : 1.0f;
+  stf(out, (size_t)r * ldo + c, v * v * w);
 }
 
 template <typename T>
@@ -49,11 +69,21 @@ __global__ void softcap_k(const T* __restrict__ y, int ld, float* __restrict__ o
 
 extern "C" {
 
-int p2p_sm_glu_act(const void* gu, int ld, void* out, int ldo, int R, int F, int f32,
+int p2p_sm_glu_act(const void* gu, int ld, void* out, int ldo, int R, int F, int act, int f32,
                    hipStream_t st) {
   if (R <= 0) return 0;
   dim3 g((F + 255) / 256, R), b(256);
-  SM_DISPATCH_T(f32, hipLaunchKernelGGL(glu_act_k<T>, g, b, 0, st, (const T*)gu, ld, (T*)out, ldo, F));
+  SM_DISPATCH_T(f32, hipLaunchKernelGGL(glu_act_k<T>, g, b, 0, st, (const T*)gu, ld, (T*)out, ldo, F,
+                                         act));
+  return (int)hipGetLastError();
+}
+
+int p2p_sm_relu2_gate(const void* u, int ld, const void* gt, int ldg, void* out, int ldo, int R,
+                      int F, int f32, hipStream_t st) {
+  if (R <= 0 || F <= 0) return 0;
+  dim3 g((F + 255) / 256, R), b(256);
+  SM_DISPATCH_T(f32, hipLaunchKernelGGL(relu2_gate_k<T>, g, b, 0, st, (const T*)u, ld,
+                                         (const T*)gt, ldg, (T*)out, ldo, F));
   return (int)hipGetLastError();
 }
 

@@ -3,16 +3,18 @@
 // not take).
 //
 // qk_norm_rope_store_k: one projection buffer holds q (H heads x D) | k (G x D) | v (G x V) of a
-// row.  q and k are RMS-normalised with one mean square per row (heads not separated) and
-// weighted, and the channel pairs (2i, 2i+1), i < nrot, of every head are turned by the angle
-// pos * inv_freq[i]:
+// row.  q and k are RMS-normalised and weighted -- with one mean square per row (heads not
+// separated, a weight per channel of the row) or, `per_head`, one per head and a weight of D
+// channels that the heads share -- and nrot channel pairs of every head, (2i, 2i+1) or, `half`,
+// (i, i + nrot), are turned by the angle pos * inv_freq[i]:
 // (a, b) -> (a cos - b sin, b cos + a sin).  q goes to its own buffer, k | v to the row of the
-// paged pool that the token owns.  Norm, angle and rotation are fp32.
+// paged pool that the token owns; a layer that reads another layer's keys and values passes no
+// pool and only its queries are prepared.  Norm, angle and rotation are fp32.
 //
 // window_attn_k: pool row = [k of G heads | v of G heads]; query head h reads key/value head
 // h / (H/G).  Causal sliding window: position i sees j with 0 <= i - j < win.  The softmax
 // denominator holds one more term exp(sink_h) that adds nothing to the numerator: the running
-// maximum starts at sink_h and the running sum at 1.  One block per (query row, key/value head): the
+// maximum starts at sink_h and the running sum at 1 (without a sink: an ordinary softmax).  One block per (query row, key/value head): the
 // heads of the group share the key and value tiles, which stream through LDS with an online
 // softmax.
 #include "common.h"
@@ -24,50 +26,62 @@ qk_norm_rope_store_k(const T* __restrict__ proj, int ldp, int H, int G, int D, i
                      const float* __restrict__ qw, const float* __restrict__ kw,
                      const float* __restrict__ inv_freq, int nrot, const int* __restrict__ pos,
                      const int* __restrict__ cache_rows, T* __restrict__ pool, float eps,
-                     T* __restrict__ q_out, int ldq) {
+                     T* __restrict__ q_out, int ldq, int per_head, int half) {
   __shared__ float red[16];
   const int r = blockIdx.x;
   const int nq = H * D, nk = G * D, nv = G * V;
+  const int heads = pool ? H + G : H;     // without a pool only the queries are prepared
   const T* row = proj + (size_t)r * ldp;
-  float sq = 0.0f, sk = 0.0f;
-  for (int i = threadIdx.x; i < nq; i += blockDim.x) {
-    float v = ldf(row, i);
-    sq += v * v;
+  float rq = 0.0f, rk = 0.0f;
+  if (!per_head) {
+    float sq = 0.0f, sk = 0.0f;
+    for (int i = threadIdx.x; i < nq; i += blockDim.x) {
+      float v = ldf(row, i);
+      sq += v * v;
+    }
+    if (pool)
+      for (int i = threadIdx.x; i < nk; i += blockDim.x) {
+        float v = ldf(row, nq + i);
+        sk += v * v;
+      }
+    sq = block_sum(sq, red);
+    sk = block_sum(sk, red);
+    rq = 1.0f / sqrtf(sq / (float)nq + eps);
+    rk = 1.0f / sqrtf(sk / (float)nk + eps);
   }
-  for (int i = threadIdx.x; i < nk; i += blockDim.x) {
-    float v = ldf(row, nq + i);
-    sk += v * v;
-  }
-  sq = block_sum(sq, red);
-  sk = block_sum(sk, red);
-  const float rq = 1.0f / sqrtf(sq / (float)nq + eps), rk = 1.0f / sqrtf(sk / (float)nk + eps);
   const float p = (float)pos[r];
-  const int D2 = (D + 1) / 2;
-  T* crow = pool + (size_t)cache_rows[r] * (nk + nv);
+  T* crow = pool ? pool + (size_t)cache_rows[r] * (nk + nv) : nullptr;
   T* qrow = q_out + (size_t)r * ldq;
-  // pairs of q, then pairs of k
-  for (int idx = threadIdx.x; idx < (H + G) * D2; idx += blockDim.x) {
-    int hh = idx / D2, j = idx % D2;
-    bool isq = hh < H;
-    int c = (isq ? hh : hh - H) * D + 2 * j;        // channel within q or k
-    bool two = 2 * j + 1 < D;
-    const float* w = isq ? qw : kw;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  // one wavefront per head: q heads, then k heads
+  for (int hh = wave; hh < heads; hh += nw) {
+    const bool isq = hh < H;
+    const int hd = isq ? hh : hh - H;
+    const T* src = row + (isq ? 0 : nq) + hd * D;
+    const float* w = (isq ? qw : kw) + (per_head ? 0 : hd * D);
+    T* dst = (isq ? qrow : crow) + hd * D;
     float rs = isq ? rq : rk;
-    int off = isq ? 0 : nq;
-    float a = ldf(row, off + c) * rs * w[c];
-    float b = two ? ldf(row, off + c + 1) * rs * w[c + 1] : 0.0f;
-    if (j < nrot) {
+    if (per_head) {
+      float ss = 0.0f;
+      for (int i = lane; i < D; i += 64) {
+        float v = ldf(src, i);
+        ss += v * v;
+      }
+      ss = wave_sum(ss);
+      rs = 1.0f / sqrtf(ss / (float)D + eps);
+    }
+    for (int j = lane; j < nrot; j += 64) {
+      int ca = half ? j : 2 * j, cb = half ? j + nrot : 2 * j + 1;
+      float a = ldf(src, ca) * rs * w[ca], b = ldf(src, cb) * rs * w[cb];
       float sn, cs;
       sincosf(p * inv_freq[j], &sn, &cs);
-      float a2 = a * cs - b * sn, b2 = b * cs + a * sn;
-      a = a2;
-      b = b2;
+      stf(dst, ca, a * cs - b * sn);
+      stf(dst, cb, b * cs + a * sn);
     }
-    T* dst = isq ? qrow : crow;
-    stf(dst, c, a);
-    if (two) stf(dst, c + 1, b);
+    for (int c = 2 * nrot + lane; c < D; c += 64) stf(dst, c, ldf(src, c) * rs * w[c]);
   }
-  for (int i = threadIdx.x; i < nv; i += blockDim.x) crow[nk + i] = row[nq + nk + i];
+  if (pool)
+    for (int i = threadIdx.x; i < nv; i += blockDim.x) crow[nk + i] = row[nq + nk + i];
 }
 
 #define WA_TK 32       // keys per tile at most
@@ -98,8 +112,8 @@ window_attn_k(const T* __restrict__ q, int ldq, const T* __restrict__ pool,
   for (int idx = tid; idx < HG * D; idx += WA_THREADS)
     sq[idx] = ldf(q, (size_t)r * ldq + (size_t)h0 * D + idx);
   if (tid < HG) {
-    sm_[tid] = sink[h0 + tid];
-    sl[tid] = 1.0f;
+    sm_[tid] = sink ? sink[h0 + tid] : -1e30f;   // no sink: an ordinary softmax
+    sl[tid] = sink ? 1.0f : 0.0f;
   }
   float acc[WA_ACC];
 #pragma unroll
@@ -180,12 +194,14 @@ extern "C" {
 int p2p_sm_qk_norm_rope_store(const void* proj, int ldp, int H, int G, int D, int V,
                               const float* qw, const float* kw, const float* inv_freq, int nrot,
                               const int* pos, const int* cache_rows, void* pool, float eps,
-                              void* q_out, int ldq, int R, int f32, hipStream_t st) {
+                              void* q_out, int ldq, int R, int per_head, int half, int f32,
+                              hipStream_t st) {
   if (R <= 0) return 0;
   if (H < 1 || G < 1 || D < 1 || V < 1 || nrot < 0 || 2 * nrot > D) return (int)hipErrorInvalidValue;
   SM_DISPATCH_T(f32, hipLaunchKernelGGL(qk_norm_rope_store_k<T>, dim3(R), dim3(256), 0, st,
                                          (const T*)proj, ldp, H, G, D, V, qw, kw, inv_freq, nrot,
-                                         pos, cache_rows, (T*)pool, eps, (T*)q_out, ldq));
+                                         pos, cache_rows, (T*)pool, eps, (T*)q_out, ldq, per_head,
+                                         half));
   return (int)hipGetLastError();
 }
 

@@ -72,8 +72,9 @@ window_attn_mfma_k(const bf16* __restrict__ q, int ldq, const bf16* __restrict__
   }
   __syncthreads();
 
-  float m_run = pvalid ? (first ? sink[ph] : -1e30f) : 0.0f;
-  float l_part = (pvalid && quad == 0 && first) ? 1.0f : 0.0f;
+  const bool sunk = first && sink != nullptr;   // no sink: an ordinary softmax
+  float m_run = pvalid ? (sunk ? sink[ph] : -1e30f) : 0.0f;
+  float l_part = (pvalid && quad == 0 && sunk) ? 1.0f : 0.0f;
   f32x4 acc[NT];
 #pragma unroll
   for (int t = 0; t < NT; t++) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};

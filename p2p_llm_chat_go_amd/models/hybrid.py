@@ -8,6 +8,8 @@ is wrapped around the residual stream,
     "gated_post"  x <- x + norm(f(x) * sigmoid(R x + b))     no norm on the way in; the norm
                                                              on the way out is taken in
                                                              equal parts of the vector
+    "parallel"    x <- x + mixer(u) + ff(u),  u = norm(x)    one norm per layer feeds both
+                                                             sublayers
 
 and whether learned absolute positions are added to the token embedding.  Mixers:
 
@@ -23,6 +25,13 @@ and whether learned absolute positions are added to the token embedding.  Mixers
   ``gated_delta``       gated delta rule: short causal convolutions + silu on q, k, v, unit
                         keys, a per-channel decay and a write that corrects what the key reads;
   ``hgrn2``             gated linear attention: the write strength is 1 - forget gate;
+  ``mlstm``             matrix memory of the xLSTM: exponential input gate, sigmoid forget gate,
+                        both in the log domain under a running maximum, and a normaliser state;
+  ``attention``         causal grouped-query attention with an ordinary softmax: RMS norm of
+                        every query / key head (one weight shared by the heads), rotary
+                        positions on channel pairs (i, i + dims/2) with optional stretching of
+                        the long wavelengths; a layer may read an earlier layer's keys and
+                        values (``kv_from``) instead of projecting its own;
   ``parallel``          two mixers side by side on the same input, summed with fixed scales.
 
 Feed-forwards: ``dense`` (silu-gated, or the clamped gated unit when the config gives a
@@ -31,7 +40,9 @@ limit) and ``moe`` (sigmoid router, choice limited to the best groups of experts
 "Regesun" stacks the first three mixers in the sandwich form with learned positions;
 "Rotutar" stacks ``parallel`` (window attention beside the gated delta rule) and ``hgrn2``
 layers in the gated post-norm form, without positions other than the rotation, and caps
-its logits with a tanh.  A checkpoint is a ``config.json`` whose ``architecture`` names the
+its logits with a tanh.  "Futetar" stacks ``mlstm`` and ``attention`` layers in the parallel form
+(norm weights stored around zero), with gelu-gated dense feed-forwards and mixtures of
+squared-relu experts behind a softmax router.  A checkpoint is a ``config.json`` whose ``architecture`` names the
 design and one safetensors file (``load_dir``).
 
 One ``forward`` serves every step: a flat list of token rows cut into entries (portions of
@@ -65,11 +76,18 @@ class LayerSpec:
 
 @dataclasses.dataclass(frozen=True)
 class Design:
-    block: str                # how sublayers sit on the residual stream: "sandwich" | "gated_post"
+    block: str                # how sublayers sit on the residual stream: "sandwich" | "gated_post" | "parallel"
     positions: str | None     # "learned": a position table is added to the embedding
+    norm_offset: float = 0.0  # block and final norm weights are stored minus this (1: around zero)
+    ff: tuple = ()            # (config kind, FEEDFORWARDS key) where the two differ
+
+    def ff_key(self, kind: str) -> str:
+        return dict(self.ff).get(kind, kind)
 
 
-DESIGNS = {"Regesun": Design("sandwich", "learned"), "Rotutar": Design("gated_post", None)}
+DESIGNS = {"Regesun": Design("sandwich", "learned"), "Rotutar": Design("gated_post", None),
+           "Futetar": Design("parallel", None, norm_offset=1.0,
+                             ff=(("dense", "dense_gelu"), ("moe", "moe_softmax")))}
 NO_POS_LIMIT = 1 << 30
 
 
@@ -110,7 +128,7 @@ class HybridConfig:
         for L in layers:
             if L.kind not in MIXERS:
                 raise KeyError("unknown mixer %r (known: %s)" % (L.kind, ", ".join(sorted(MIXERS))))
-            if L.mlp is not None and L.mlp.get("kind", "dense") not in FEEDFORWARDS:
+            if L.mlp is not None and DESIGNS[design].ff_key(L.mlp.get("kind", "dense")) not in FEEDFORWARDS:
                 raise KeyError("unknown feed-forward kind %r" % L.mlp.get("kind"))
         eos = c.get("eos_token_id", ())
         eos = tuple(eos) if isinstance(eos, (list, tuple)) else (int(eos),)
@@ -405,9 +423,13 @@ class LatentAttention(Mixer):
 class WindowAttention(Mixer):
     """Grouped-query attention with cached keys and values (``ops.seqmix.window_attn``)."""
     kind = "window_attention"
+    PER_HEAD = False   # query / key norm per head with one weight of D channels, or over the row
+    HALF = False       # rotated pairs (i, i + dims/2) or (2i, 2i+1)
+    SINK = True        # softmax denominator with a learned per-head sink
 
     def _dims(self):
         s = self.spec
+        self.kv_from = int(s["kv_from"]) if s.get("kv_from") is not None else None
         self.H, self.D, self.V = int(s["heads"]), int(s["dim"]), int(s["vdim"])
         self.G = int(s.get("kv_heads", self.H))
         self.win = int(s["mask"]["size"]) if s.get("mask") else 1 << 30
@@ -415,6 +437,7 @@ class WindowAttention(Mixer):
         rot = s.get("rot")
         self.rot_dims = int(rot["dims"]) if rot else 0
         self.rot_base = float(rot["base"]) if rot else 1.0
+        self.rot_scaling = dict(rot["scaling"]) if rot and rot.get("scaling") else None
         if self.H % self.G or self.rot_dims % 2 or self.rot_dims > self.D:
             raise ValueError("window_attention: %d heads / %d kv heads / %d rotated of %d channels"
                              % (self.H, self.G, self.rot_dims, self.D))
@@ -423,28 +446,94 @@ class WindowAttention(Mixer):
     def tensor_shapes(self):
         self._dims()
         H, G, D, V, W = self.H, self.G, self.D, self.V, self.width
-        return {"q": (H * D, W), "k": (G * D, W), "v": (G * V, W), "q.norm": (H * D,),
-                "k.norm": (G * D,), "sink": (H,), "o": (W, H * V)}
+        d = {"q": (H * D, W), "q.norm": (D,) if self.PER_HEAD else (H * D,), "o": (W, H * V)}
+        if self.kv_from is None:   # a layer that borrows keys and values has no tensors of them
+            d.update({"k": (G * D, W), "v": (G * V, W), "k.norm": (D,) if self.PER_HEAD else (G * D,)})
+        if self.SINK:
+            d["sink"] = (H,)
+        return d
 
     def load(self, get, dtype, dev):
         self._dims()
-        self.w_in = torch.cat([get("q"), get("k"), get("v")], 0).to(dev, dtype).contiguous()
-        self.qnorm, self.knorm, self.sink = (_vec(get(k), dev) for k in ("q.norm", "k.norm", "sink"))
-        self.inv_freq = sm.rope_inv_freq(self.rot_base, self.rot_dims, dev)
+        own = self.kv_from is None
+        names = ("q", "k", "v") if own else ("q",)
+        self.w_in = torch.cat([get(k) for k in names], 0).to(dev, dtype).contiguous()
+        self.qnorm = _vec(get("q.norm"), dev)
+        self.knorm = _vec(get("k.norm"), dev) if own else None
+        self.sink = _vec(get("sink"), dev) if self.SINK else None
+        self.inv_freq = sm.rope_inv_freq(self.rot_base, self.rot_dims, dev, self.rot_scaling)
         self.wo = get("o").to(dev, dtype).contiguous()
 
     def cache_spec(self):
-        return ("paged", self.G * (self.D + self.V))
+        return ("paged", self.G * (self.D + self.V)) if self.kv_from is None else None
+
+    def shares_cache_with(self, other) -> bool:
+        """Whether this layer can read the keys and values that ``other`` leaves in its pool."""
+        return (isinstance(other, WindowAttention) and other.kv_from is None
+                and (other.G, other.D, other.V, other.PER_HEAD, other.HALF)
+                == (self.G, self.D, self.V, self.PER_HEAD, self.HALF)
+                and (other.rot_dims, other.rot_base, other.rot_scaling)
+                == (self.rot_dims, self.rot_base, self.rot_scaling))
 
     def mix(self, proj, b, cache, layer, out, out_scale=1.0):
         H, G, D, V = self.H, self.G, self.D, self.V
-        pool = cache.paged[layer]
+        own = self.kv_from is None
+        pool = cache.paged[layer if own else self.kv_from]
         q = torch.empty(b.R, H * D, device=proj.device, dtype=proj.dtype)
         sm.qk_norm_rope_store(proj, H, G, D, V, self.qnorm, self.knorm, self.inv_freq, b.pos,
-                              b.cache_rows, pool, self.eps, q)
+                              b.cache_rows, pool if own else None, self.eps, q,
+                              per_head=self.PER_HEAD, half=self.HALF)
         units = b.units(sm.window_rows_per_wave(H // G)) if sm.window_mfma_ok(q, pool, D, V) else None
         sm.window_attn(q, pool, b.block_tables, b.row_ent, b.pos, self.sink, self.scale, self.win,
                        out, PAGE, H, G, D, V, units=units, max_keys=b.max_keys, out_scale=out_scale)
+        return out
+
+
+class Attention(WindowAttention):
+    """Causal grouped-query attention with an ordinary softmax: per-head query / key norm,
+    rotation of the pairs (i, i + dims/2) with optional stretching of long wavelengths
+    (``rot.scaling``), no sink; ``mask`` (a window) stays optional.  ``kv_from: j`` reads layer
+    j's keys and values as its cache holds them and projects only queries."""
+    kind = "attention"
+    PER_HEAD, HALF, SINK = True, True, False
+
+
+class MLSTM(Mixer):
+    """Matrix memory of the xLSTM (``ops.seqmix.mlstm_scan``): per head a D x V memory and a
+    normaliser, written through an exponential input gate and decayed by a sigmoid forget gate
+    whose pre-activations are capped by ``gate_cap * tanh(. / gate_cap)``; head norm, a weight
+    per channel and a sigmoid output gate on the way out."""
+    kind = "mlstm"
+
+    def _dims(self):
+        s = self.spec
+        self.H, self.D, self.V = int(s["heads"]), int(s["dim"]), int(s["vdim"])
+        self.cap = float(s["gate_cap"])
+        if self.cap <= 0:
+            raise ValueError("mlstm: gate cap %g" % self.cap)
+        self.n_mid = self.H * self.V
+
+    def tensor_shapes(self):
+        self._dims()
+        H, D, V, W = self.H, self.D, self.V, self.width
+        return {"q": (H * D, W), "k": (H * D, W), "v": (H * V, W), "g": (H * V, W), "o": (W, H * V),
+                "norm": (H * V,), "i": (H, W), "i.b": (H,), "f": (H, W), "f.b": (H,)}
+
+    def load(self, get, dtype, dev):
+        self._dims()
+        # one projection for everything that reads the layer input: q | k | v | gate | i | f
+        self.w_in = torch.cat([get(k) for k in ("q", "k", "v", "g", "i", "f")], 0).to(dev, dtype).contiguous()
+        self.bi, self.bf, self.normw = (_vec(get(k), dev) for k in ("i.b", "f.b", "norm"))
+        self.wo = get("o").to(dev, dtype).contiguous()
+
+    def cache_spec(self):
+        # column V of the memory holds the normaliser; m is the running maximum of the log gates
+        return ("state", {"S": (self.H, self.D, self.V + 1), "m": (self.H,)})
+
+    def mix(self, proj, b, cache, layer, out, out_scale=1.0):
+        st = cache.state[layer]
+        sm.mlstm_scan(proj, self.bi, self.bf, self.cap, self.normw, st["S"], st["m"], b.ent,
+                      b.ent_host, out, self.H, self.D, self.V, self.eps, out_scale=out_scale)
         return out
 
 
@@ -582,16 +671,23 @@ class Parallel(Mixer):
 
 
 MIXERS = {c.kind: c for c in (GeneralDelta, Mamba2, LatentAttention, WindowAttention, GatedDelta,
-                              HGRN2, Parallel)}
+                              HGRN2, Parallel, Attention, MLSTM)}
 
 
 class DenseFF:
     """Gated feed-forward W_down(act(W_gate h) * W_up h): silu-gated, or with a ``limit`` in its
-    config the clamped unit of ``ops.seqmix.ff_act``."""
+    config the clamped unit of ``ops.seqmix.ff_act``.
+
+    Every feed-forward offers two ways in: ``forward(h)``, or for a layer that runs the
+    projections of its input and the output projections of its sublayers as one product each:
+    ``w_in`` (rows that read the layer input, or None), ``fill(proj, h, mid)`` (writes the
+    input of the output projection, [R, n_mid]; may return a part of the result that is added
+    separately) and ``w_out`` [width, n_mid]."""
+    ACT = "silu"
 
     def __init__(self, spec: dict, width: int):
         self.spec, self.width = spec, width
-        self.F = int(spec["ff"])
+        self.F = self.n_mid = int(spec["ff"])
         self.limit = float(spec["limit"]) if spec.get("limit") is not None else None
 
     def tensor_shapes(self):
@@ -600,15 +696,19 @@ class DenseFF:
     def load(self, get, dtype, dev):
         self.w_gu = torch.cat([get("gate"), get("up")], 0).to(dev, dtype).contiguous()
         self.w_in = self.w_gu
-        self.w_down = get("down").to(dev, dtype).contiguous()
+        self.w_down = self.w_out = get("down").to(dev, dtype).contiguous()
+
+    def fill(self, gu, h, mid):
+        if self.limit is None:
+            sm.glu_act(gu, mid, self.ACT)
+        else:
+            sm.ff_act(gu, mid, self.limit)
+        return None
 
     def forward_proj(self, gu):
         """gu = [gate | up] projections of the input."""
         act = torch.empty(gu.shape[0], self.F, device=gu.device, dtype=gu.dtype)
-        if self.limit is None:
-            sm.glu_act(gu, act)
-        else:
-            sm.ff_act(gu, act, self.limit)
+        self.fill(gu, None, act)
         return F.linear(act, self.w_down)
 
     def forward(self, h):
@@ -620,7 +720,11 @@ class MoEFF:
     the best groups of experts (``ops.seqmix.group_route``); the chosen experts' scores weight
     their outputs without rescaling.  The expert products run grouped over the routed rows
     (``ops.seqmix.expert_gemm``)."""
-    w_in = None   # the router and the grouped products read the input themselves
+    w_in = w_out = None   # the router and the grouped products read the input themselves
+    n_mid = 0
+
+    def fill(self, proj, h, mid):
+        return self.forward(h)
 
     def __init__(self, spec: dict, width: int):
         self.spec, self.width = spec, width
@@ -673,21 +777,112 @@ class MoEFF:
         return sm.expert_combine(y, wts, out)
 
 
-FEEDFORWARDS = {"dense": DenseFF, "moe": MoEFF}
+class GeluFF(DenseFF):
+    """W_down(gelu(W_gate h) * W_up h) with the tanh form of gelu."""
+    ACT = "gelu_tanh"
+
+
+class SoftmaxMoEFF:
+    """Mixture of ungated squared-relu experts, W_down relu(W_up h)^2, behind a softmax router
+    (``ops.seqmix.group_route``): scores s = softmax over all router outputs; the choice is made
+    on s + ``correction``, limited to the ``groups.keep`` groups of neighbouring experts whose
+    best choice score is largest; the weights are the chosen s, not rescaled.  The last
+    ``router.identity`` router outputs stand for experts without tensors that hand their input
+    back.  An optional shared expert of the same form runs for every token, weighted by
+    sigmoid(W_sg h); its products ride on the layer's input and output products."""
+
+    def __init__(self, spec: dict, width: int):
+        self.spec, self.width = spec, width
+        r = spec["router"]
+        self.E, self.top = int(r["experts"]), int(r["top"])          # experts with tensors
+        self.ident = int(r.get("identity", 0))
+        self.EA = self.E + self.ident                                 # router outputs
+        g = r.get("groups") or {}
+        self.groups, self.keep = int(g.get("count", 1)), int(g.get("keep", g.get("count", 1)))
+        self.F = int(spec["expert"]["ff"])
+        self.Fs = self.n_mid = int(spec["shared"]["ff"]) if spec.get("shared") else 0
+        per = self.EA // max(1, self.groups)
+        if self.groups < 1 or self.EA % self.groups or not 1 <= self.keep <= self.groups \
+                or not 1 <= self.top <= self.keep * per or self.E < 0 or self.ident < 0:
+            raise ValueError("moe: %d + %d experts in %d groups, %d kept, %d chosen"
+                             % (self.E, self.ident, self.groups, self.keep, self.top))
+
+    def tensor_shapes(self):
+        d = {"router": (self.EA, self.width), "correction": (self.EA,)}
+        for e in range(self.E):
+            d.update({"e%d.up" % e: (self.F, self.width), "e%d.down" % e: (self.width, self.F)})
+        if self.Fs:
+            d.update({"shared.up": (self.Fs, self.width), "shared.down": (self.width, self.Fs),
+                      "shared.sg": (1, self.width)})
+        return d
+
+    def load(self, get, dtype, dev):
+        self.wr = get("router").to(dev).float().contiguous()
+        self.corr = _vec(get("correction"), dev)
+        self.w_up = self.w_dn = None
+        if self.E:
+            self.w_up = torch.stack([get("e%d.up" % e) for e in range(self.E)]).to(dev, dtype).contiguous()
+            self.w_dn = torch.stack([get("e%d.down" % e) for e in range(self.E)]).to(dev, dtype).contiguous()
+        self.w_in = self.w_out = None
+        if self.Fs:
+            self.w_in = torch.cat([get("shared.up"), get("shared.sg")], 0).to(dev, dtype).contiguous()
+            self.w_out = get("shared.down").to(dev, dtype).contiguous()
+
+    def routed(self, h):
+        R, top, dev = h.shape[0], self.top, h.device
+        ids = torch.empty(R, top, device=dev, dtype=torch.int32)
+        wts = torch.empty(R, top, device=dev, dtype=torch.float32)
+        cnt = torch.empty(self.EA, device=dev, dtype=torch.int32)
+        rows = torch.empty(self.EA, R * top, device=dev, dtype=torch.int32)
+        sm.group_route(h, self.wr, top, self.groups, self.keep, ids, wts, cnt, rows,
+                       score="softmax", corr=self.corr, group_score="max")
+        y = torch.empty(R * top, self.width, device=dev, dtype=h.dtype)
+        if self.E:
+            act = torch.empty(R * top, self.F, device=dev, dtype=h.dtype)
+            sm.expert_gemm(h, top, self.w_up, cnt, rows, act, R * top, relu2=True)
+            sm.expert_gemm(act, 1, self.w_dn, cnt, rows, y, R * top)
+        out = torch.empty(R, self.width, device=dev, dtype=h.dtype)
+        return sm.expert_combine(y, wts, out, ids=ids if self.ident else None, n_real=self.E, x=h)
+
+    def fill(self, proj, h, mid):
+        if self.Fs:
+            sm.relu2_gate(proj, proj[:, self.Fs:self.Fs + 1], mid)
+        return self.routed(h)
+
+    def forward(self, h):
+        y = self.routed(h)
+        if self.Fs:
+            proj = F.linear(h, self.w_in)
+            mid = torch.empty(h.shape[0], self.Fs, device=h.device, dtype=h.dtype)
+            sm.relu2_gate(proj, proj[:, self.Fs:self.Fs + 1], mid)
+            y = y + F.linear(mid, self.w_out)
+        return y
+
+
+FEEDFORWARDS = {"dense": DenseFF, "moe": MoEFF, "dense_gelu": GeluFF, "moe_softmax": SoftmaxMoEFF}
 
 
 # ---------------------------------------------------------------------------- weights
 class HybridLayer:
     def __init__(self, spec: LayerSpec, cfg: HybridConfig):
         self.block = cfg.traits.block
+        self.norm_offset = cfg.traits.norm_offset
         self.mixer = MIXERS[spec.kind](spec.mixer, cfg.width, cfg.eps)
-        self.ff = FEEDFORWARDS[spec.mlp.get("kind", "dense")](spec.mlp, cfg.width) \
+        self.ff = FEEDFORWARDS[cfg.traits.ff_key(spec.mlp.get("kind", "dense"))](spec.mlp, cfg.width) \
             if spec.mlp is not None else None
+        # parallel: the layer's input and output products (mixer and feed-forward together)
+        self.w_in_all = self.w_out_all = None
         self.norm1 = self.norm1b = self.ls1 = self.norm2 = self.norm2b = self.ls2 = None
         # gated_post: the gates' projections ride on the sublayers' input products
         self.w_in1 = self.w_in2 = self.rg1b = self.rg2b = None
 
     def tensor_shapes(self, W):
+        if self.block == "parallel":
+            d = {"norm1": (W,)}
+            d.update({"mix." + k: s for k, s in self.mixer.tensor_shapes().items()})
+            if self.ff is not None:
+                d.update({"mlp." + k: s for k, s in self.ff.tensor_shapes().items()})
+            return d
         gated = self.block == "gated_post"
         d = {"norm1": (W,), "rg1": (W, W), "rg1.b": (W,)} if gated else \
             {"norm1": (W,), "norm1b": (W,), "ls1": (W,)}
@@ -702,6 +897,18 @@ class HybridLayer:
         self.mixer.load(lambda k: sd[p + "mix." + k], dtype, dev)
         if self.ff is not None:
             self.ff.load(lambda k: sd[p + "mlp." + k], dtype, dev)
+        if self.block == "parallel":
+            if self.mixer.w_in is None or self.mixer.wo is None:
+                raise ValueError("mixer %r cannot share the layer's products" % self.mixer.kind)
+            self.norm1 = (_vec(sd[p + "norm1"], dev) + self.norm_offset).contiguous()
+            ins, outs = [self.mixer.w_in], [self.mixer.wo]
+            if self.ff is not None and self.ff.w_in is not None:
+                ins.append(self.ff.w_in)
+            if self.ff is not None and self.ff.n_mid:
+                outs.append(self.ff.w_out)
+            self.w_in_all = torch.cat(ins, 0).contiguous() if len(ins) > 1 else ins[0]
+            self.w_out_all = torch.cat(outs, 1).contiguous() if len(outs) > 1 else outs[0]
+            return
         if self.block == "gated_post":
             if self.mixer.w_in is None:
                 raise ValueError("mixer %r cannot share its input product with a gate" % self.mixer.kind)
@@ -745,13 +952,14 @@ class HybridWeights:
                 raise ValueError("tensor %r has shape %s, the config gives %s" % (k, tuple(sd[k].shape), s))
         self.embed = sd["embed"].to(dev, dtype).contiguous()
         self.pos = sd["pos"].to(dev, dtype).contiguous() if cfg.traits.positions else None
-        self.final_norm = _vec(sd["final.norm"], dev)
+        self.final_norm = (_vec(sd["final.norm"], dev) + cfg.traits.norm_offset).contiguous()
         self.head = sd["head"].to(dev, dtype).contiguous()
         self.layers = []
         for i, spec in enumerate(cfg.layers):
             L = HybridLayer(spec, cfg)
             L.load(sd, "l%d." % i, dtype, dev)
             self.layers.append(L)
+        check_shared_caches([L.mixer for L in self.layers])
 
     @classmethod
     def random(cls, cfg: HybridConfig, device="cuda", seed: int = 0, dtype=torch.bfloat16):
@@ -759,6 +967,17 @@ class HybridWeights:
 
     def cache_specs(self) -> list:
         return [L.mixer.cache_spec() for L in self.layers]
+
+
+def check_shared_caches(mixers: list):
+    """A layer that reads another layer's keys and values names an earlier layer that keeps a
+    pool of the same shape, filled the same way."""
+    for i, m in enumerate(mixers):
+        j = getattr(m, "kv_from", None)
+        if j is None:
+            continue
+        if not 0 <= j < i or not m.shares_cache_with(mixers[j]):
+            raise ValueError("layer %d cannot read the keys and values of layer %d" % (i, j))
 
 
 def random_state_dict(cfg: HybridConfig, seed: int = 0) -> dict:
@@ -772,8 +991,12 @@ def random_state_dict(cfg: HybridConfig, seed: int = 0) -> dict:
             t = torch.randn(*s, generator=g) / (s[1] ** 0.5 if k not in ("embed", "pos") else 1.0)
         elif leaf.endswith("conv"):
             t = torch.randn(*s, generator=g) * 0.5
-        elif leaf.endswith(("norm1", "norm2", "norm1b", "norm2b", ".norm")) or k == "final.norm":
+        elif leaf in ("norm1", "norm2", "norm1b", "norm2b") or k == "final.norm":
+            t = (1.0 - cfg.traits.norm_offset) + 0.1 * torch.randn(*s, generator=g)
+        elif leaf.endswith(".norm"):
             t = 1.0 + 0.1 * torch.randn(*s, generator=g)
+        elif leaf.endswith("correction"):
+            t = 0.05 * torch.randn(*s, generator=g)
         elif leaf.endswith("lower"):
             t = torch.rand(*s, generator=g) * 0.9
         elif leaf in ("ls1", "ls2"):
@@ -815,6 +1038,8 @@ class HybridModel:
             raise ValueError("position %d exceeds the model's %d positions" % (b.max_pos, cfg.max_pos))
         if cfg.traits.block == "gated_post":
             return self._forward_gated_post(b, layer_out)
+        if cfg.traits.block == "parallel":
+            return self._forward_parallel(b, layer_out)
         x = torch.empty(b.R, cfg.width, device=self.device, dtype=torch.float32)
         sm.embed_pos(w.embed, w.pos, b.ids, b.pos, x)
         h = torch.empty(b.R, cfg.width, device=self.device, dtype=self.dtype)
@@ -869,6 +1094,33 @@ class HybridModel:
                     n = L.ff.w_in.shape[0]
                     f, gate = L.ff.forward_proj(proj[:, :n]), proj[:, n:]
                 sm.gate_norm_add(x, f, gate, L.rg2b, L.norm2, parts, eps, next_out=nxt)
+            if layer_out is not None:
+                layer_out.append(x.clone())
+        if b.n_out == 0:
+            return None
+        return self._logits(x, b)
+
+    def _forward_parallel(self, b: StepBatch, layer_out=None):
+        """x <- x + mixer(u) + ff(u) with u = norm(x): one product forms every projection of u
+        (the mixer's and the feed-forward's), the sublayers write the inputs of their output
+        projections side by side into one buffer, and one product with the joined output
+        weights gives mixer(u) + ff(u) summed in its fp32 accumulator.  What a feed-forward
+        computes apart from that (routed experts) is added in the same fp32 pass that updates
+        the residual and forms the next layer's u."""
+        cfg, w = self.cfg, self.w
+        x = torch.empty(b.R, cfg.width, device=self.device, dtype=torch.float32)
+        sm.embed_rows(w.embed, b.ids, x, None)
+        h = torch.empty(b.R, cfg.width, device=self.device, dtype=self.dtype)
+        sm.rmsnorm(x, w.layers[0].norm1, cfg.eps, h)
+        for i, L in enumerate(w.layers):
+            proj = F.linear(h, L.w_in_all)
+            nm, mm = L.mixer.w_in.shape[0], L.mixer.n_mid
+            mid = torch.empty(b.R, L.w_out_all.shape[1], device=self.device, dtype=self.dtype)
+            L.mixer.mix(proj[:, :nm], b, self.cache, i, mid[:, :mm])
+            extra = L.ff.fill(proj[:, nm:], h, mid[:, mm:]) if L.ff is not None else None
+            y = F.linear(mid, L.w_out_all)
+            nxt = w.layers[i + 1].norm1 if i + 1 < len(w.layers) else None
+            sm.add_norm(x, y, extra, cfg.eps, next_w=nxt, next_out=h)
             if layer_out is not None:
                 layer_out.append(x.clone())
         if b.n_out == 0:

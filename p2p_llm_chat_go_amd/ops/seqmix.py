@@ -67,13 +67,21 @@ _SIGS = {
                       c_void_p],
     "p2p_sm_gate_norm_add": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int,
                              c_int, c_int, c_float, c_void_p, c_int, c_int, c_int, c_void_p],
-    "p2p_sm_glu_act": [c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+    "p2p_sm_glu_act": [c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "p2p_sm_relu2_gate": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int,
+                          c_void_p],
+    "p2p_sm_add_norm": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_float,
+                        c_void_p, c_void_p, c_int, c_int, c_void_p],
+    "p2p_sm_mlstm_scan": [c_void_p, c_int, c_void_p, c_void_p, c_float, c_void_p, c_void_p,
+                          c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
+                          c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_float, c_float,
+                          c_int, c_void_p],
     "p2p_sm_softcap": [c_void_p, c_int, c_void_p, c_int, c_int, c_float, c_int, c_void_p],
     "p2p_sm_embed_rows": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                           c_void_p],
     "p2p_sm_qk_norm_rope_store": [c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p,
                                   c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_float,
-                                  c_void_p, c_int, c_int, c_int, c_void_p],
+                                  c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "p2p_sm_window_attn": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                            c_void_p, c_float, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int,
                            c_int, c_int, c_float, c_int, c_void_p],
@@ -96,12 +104,13 @@ _SIGS = {
                                 c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_float,
                                 c_int, c_void_p],
     "p2p_sm_group_route": [c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
-                           c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
+                           c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+                           c_int, c_void_p],
     "p2p_sm_expert_gemm": [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                            c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_int,
                            c_void_p],
     "p2p_sm_expert_combine": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
-                              c_int, c_void_p],
+                              c_void_p, c_int, c_void_p, c_int, c_int, c_void_p],
 }
 
 _lock = threading.Lock()
@@ -281,6 +290,38 @@ def norm_scale_add(x, y, w, ls, eps, next_w=None, next_out=None):
                                      _lib.ptr(ls), R, n, eps, _lib.ptr(next_w),
                                      _lib.ptr(next_out if next_w is not None else None), ldh,
                                      _f32(y), _st(x)), "norm_scale_add")
+    return x
+
+
+def add_norm(x, a, b=None, eps: float = 0.0, next_w=None, next_out=None):
+    """x += a (+ b) on the fp32 residual x, the addends summed first in fp32.  With next_w /
+    next_out also the next layer's input in the same pass:
+    next_out = x / sqrt(mean(x^2) + eps) * next_w from the updated rows."""
+    R, n = x.shape
+    if not x.is_cuda:
+        y = a[:R].float()
+        if b is not None:
+            y = y + b[:R].float()
+        x += y
+        if next_w is not None:
+            next_out[:R] = (_rms(x, eps) * next_w).to(next_out.dtype)
+        return x
+    _rows2d(a, "a")
+    assert x.dtype == torch.float32 and x.is_contiguous() and a.shape[1] == n and a.shape[0] >= R
+    ldb = 0
+    if b is not None:
+        _rows2d(b, "b")
+        assert b.shape[1] == n and b.shape[0] >= R and b.dtype == a.dtype
+        ldb = b.stride(0)
+    ldh = 0
+    if next_w is not None:
+        _vec(next_w, n, "next_w")
+        _rows2d(next_out, "next_out")
+        assert next_out.dtype == a.dtype and next_out.shape[1] == n and next_out.shape[0] >= R
+        ldh = next_out.stride(0)
+    _chk(lib().p2p_sm_add_norm(x.data_ptr(), a.data_ptr(), a.stride(0), _lib.ptr(b), ldb, R, n, eps,
+                               _lib.ptr(next_w), _lib.ptr(next_out if next_w is not None else None),
+                               ldh, _f32(a), _st(x)), "add_norm")
     return x
 
 
@@ -657,18 +698,47 @@ def gate_norm_add(x, y, g, gb, w, parts: int, eps: float, next_out=None):
     return x
 
 
-def glu_act(gu, out):
-    """[gate | up] -> silu(gate) * up."""
+GLU_ACTS = {"silu": 0, "gelu_tanh": 1}
+
+
+def glu_act(gu, out, act: str = "silu"):
+    """[gate | up] -> act(gate) * up; act: "silu", or "gelu_tanh" =
+    0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))."""
     R, F = out.shape
+    code = GLU_ACTS[act]
     if not gu.is_cuda:
         g = gu[:, :F].float()
-        out.copy_((g * torch.sigmoid(g) * gu[:, F:].float()).to(out.dtype))
+        a = g * torch.sigmoid(g) if code == 0 else \
+            0.5 * g * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (g + 0.044715 * g * g * g)))
+        out.copy_((a * gu[:, F:2 * F].float()).to(out.dtype))
         return out
     _rows2d(gu, "gu")
     _rows2d(out, "out")
-    assert gu.shape == (R, 2 * F) and gu.dtype == out.dtype
+    assert gu.shape[0] == R and gu.shape[1] >= 2 * F and gu.dtype == out.dtype
     _chk(lib().p2p_sm_glu_act(gu.data_ptr(), gu.stride(0), out.data_ptr(), out.stride(0), R, F,
-                              _f32(gu), _st(gu)), "glu_act")
+                              code, _f32(gu), _st(gu)), "glu_act")
+    return out
+
+
+def relu2_gate(u, g, out):
+    """out[r, c] = relu(u[r, c])^2 * sigmoid(g[r]): an ungated squared-relu unit weighted by one
+    gate per row (g: an [R, 1] view, or None for no gate)."""
+    R, F = out.shape
+    if not u.is_cuda:
+        v = torch.relu(u[:R, :F].float()) ** 2
+        if g is not None:
+            v = v * torch.sigmoid(g[:R, :1].float())
+        out.copy_(v.to(out.dtype))
+        return out
+    _rows2d(u, "u")
+    _rows2d(out, "out")
+    assert u.shape[0] == R and u.shape[1] >= F and u.dtype == out.dtype
+    ldg = 0
+    if g is not None:
+        assert g.dim() == 2 and g.shape[0] == R and g.dtype == u.dtype
+        ldg = g.stride(0)
+    _chk(lib().p2p_sm_relu2_gate(u.data_ptr(), u.stride(0), _lib.ptr(g), ldg, out.data_ptr(),
+                                 out.stride(0), R, F, _f32(u), _st(u)), "relu2_gate")
     return out
 
 
@@ -685,53 +755,79 @@ def softcap(y, cap: float, out):
 
 
 # ------------------------------------------------------------------ windowed attention
-def rope_inv_freq(base: float, dims: int, device) -> torch.Tensor:
-    """f_i = base^(-2i/dims), i < dims/2, evaluated in float64 and rounded to fp32."""
+def rope_inv_freq(base: float, dims: int, device, scaling: dict | None = None) -> torch.Tensor:
+    """f_i = base^(-2i/dims), i < dims/2, evaluated in float64 and rounded to fp32.
+
+    scaling = {factor, low, high, original} stretches the long wavelengths: with l = 2 pi / f,
+    f stays where l < original / high, becomes f / factor where l > original / low, and in
+    between is (1 - s) f / factor + s f with s = (original / l - low) / (high - low)."""
     i = torch.arange(dims // 2, dtype=torch.float64)
-    return torch.pow(torch.tensor(float(base), dtype=torch.float64), -2.0 * i / dims).float().to(device)
+    f = torch.pow(torch.tensor(float(base), dtype=torch.float64), -2.0 * i / dims)
+    if scaling:
+        fac, lo, hi = float(scaling["factor"]), float(scaling["low"]), float(scaling["high"])
+        orig = float(scaling["original"])
+        wl = 2.0 * math.pi / f
+        s = (orig / wl - lo) / (hi - lo) if hi != lo else torch.zeros_like(f)
+        mid = (1.0 - s) * f / fac + s * f
+        f = torch.where(wl < orig / hi, f, torch.where(wl > orig / lo, f / fac, mid))
+    return f.float().to(device)
 
 
 def qk_norm_rope_store(proj, H: int, G: int, D: int, V: int, qw, kw, inv_freq, pos, cache_rows,
-                       pool, eps: float, q_out):
+                       pool, eps: float, q_out, per_head: bool = False, half: bool = False):
     """Prepares attention inputs from one projection buffer proj = [q (H*D) | k (G*D) | v (G*V)]:
-    q and k are RMS-normalised with one mean square per row (heads not separated) and weights qw / kw,
-    then channels (2i, 2i+1), i < len(inv_freq), of every head are rotated by pos * inv_freq[i].
+    q and k are RMS-normalised and weighted -- one mean square per row (heads not separated)
+    and weights qw [H*D] / kw [G*D], or with ``per_head`` one mean square per head and weights
+    of D channels shared by the heads -- then nrot = len(inv_freq) channel pairs of every head,
+    (2i, 2i+1) or with ``half`` (i, i + nrot), are rotated by pos * inv_freq[i].
     q goes to q_out [R, H*D]; k | v go to the paged pool rows ``cache_rows`` ([tokens,
-    G*D + G*V]).  Norm, angles and the rotation are fp32."""
+    G*D + G*V]).  pool None: the layer reads another layer's keys and values, proj holds only
+    q and only q is prepared.  Norm, angles and the rotation are fp32."""
     R = q_out.shape[0]
     nq, nk, nv = H * D, G * D, G * V
     nrot = inv_freq.numel()
     if not proj.is_cuda:
         ang = (pos[:R].float()[:, None] * inv_freq[None, :])
         c, s = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+        ia = torch.arange(nrot) if half else torch.arange(0, 2 * nrot, 2)
+        ib = ia + nrot if half else ia + 1
 
-        def rot(t, heads):
-            t = t.view(R, heads, D).clone()
-            u, v = t[:, :, 0:2 * nrot:2].clone(), t[:, :, 1:2 * nrot:2].clone()
-            t[:, :, 0:2 * nrot:2] = u * c - v * s
-            t[:, :, 1:2 * nrot:2] = v * c + u * s
+        def prep(t, heads, w):
+            if per_head:
+                t = _rms(t.float().view(R, heads, D), eps) * w
+            else:
+                t = (_rms(t.float(), eps) * w).view(R, heads, D)
+            t = t.clone()
+            u, v = t[:, :, ia].clone(), t[:, :, ib].clone()
+            t[:, :, ia] = u * c - v * s
+            t[:, :, ib] = v * c + u * s
             return t.reshape(R, heads * D)
 
-        q = rot(_rms(proj[:R, :nq].float(), eps) * qw, H)
-        k = rot(_rms(proj[:R, nq:nq + nk].float(), eps) * kw, G)
-        q_out[:R] = q.to(q_out.dtype)
-        rows = cache_rows[:R].long()
-        pool[rows, :nk] = k.to(pool.dtype)
-        pool[rows, nk:] = proj[:R, nq + nk:nq + nk + nv].to(pool.dtype)
+        q_out[:R] = prep(proj[:R, :nq], H, qw).to(q_out.dtype)
+        if pool is not None:
+            rows = cache_rows[:R].long()
+            pool[rows, :nk] = prep(proj[:R, nq:nq + nk], G, kw).to(pool.dtype)
+            pool[rows, nk:] = proj[:R, nq + nk:nq + nk + nv].to(pool.dtype)
         return q_out
     _rows2d(proj, "proj")
     _rows2d(q_out, "q_out")
-    assert proj.shape[1] >= nq + nk + nv and q_out.shape[1] == nq and q_out.dtype == proj.dtype
-    assert pool.dim() == 2 and pool.is_contiguous() and pool.shape[1] == nk + nv
-    assert pool.dtype == proj.dtype
-    _vec(qw, nq, "qw")
-    _vec(kw, nk, "kw")
+    assert q_out.shape[1] == nq and q_out.dtype == proj.dtype
+    _vec(qw, D if per_head else nq, "qw")
+    if pool is not None:
+        assert proj.shape[1] >= nq + nk + nv
+        assert pool.dim() == 2 and pool.is_contiguous() and pool.shape[1] == nk + nv
+        assert pool.dtype == proj.dtype and cache_rows.dtype == torch.int32
+        _vec(kw, D if per_head else nk, "kw")
+    else:
+        assert proj.shape[1] >= nq
     assert inv_freq.dtype == torch.float32 and inv_freq.is_contiguous() and 2 * nrot <= D
-    assert pos.dtype == torch.int32 and cache_rows.dtype == torch.int32
+    assert pos.dtype == torch.int32
     _chk(lib().p2p_sm_qk_norm_rope_store(proj.data_ptr(), proj.stride(0), H, G, D, V,
-                                         qw.data_ptr(), kw.data_ptr(), inv_freq.data_ptr(), nrot,
-                                         pos.data_ptr(), cache_rows.data_ptr(), pool.data_ptr(),
-                                         eps, q_out.data_ptr(), q_out.stride(0), R, _f32(proj),
+                                         qw.data_ptr(), _lib.ptr(kw if pool is not None else None),
+                                         inv_freq.data_ptr(), nrot, pos.data_ptr(),
+                                         cache_rows.data_ptr(), _lib.ptr(pool), eps,
+                                         q_out.data_ptr(), q_out.stride(0), R,
+                                         1 if per_head else 0, 1 if half else 0, _f32(proj),
                                          _st(proj)), "qk_norm_rope_store")
     return q_out
 
@@ -759,7 +855,8 @@ def window_attn(q, pool, block_tables, row_ent, pos, sink, scale: float, win: in
     q [R, H*D] (rotated), pool [tokens, G*D + G*V] (token t of a sequence at
     block_tables[e, t // page] * page + t % page; keys first, then values), query head h reads
     key/value head h // (H/G).  out [R, H*V] = sum_j p_j v_j with
-    p = softmax over {sink_h} U {scale * q . k_j : 0 <= pos - j < win}; the sink has no value;
+    p = softmax over {sink_h} U {scale * q . k_j : 0 <= pos - j < win}; the sink has no value
+    (sink None: an ordinary softmax over the visible keys);
     the result is multiplied by out_scale before it is rounded.
     units: ``make_units(entries, window_rows_per_wave(H // G))`` on the device; with it bf16
     inputs run on the matrix cores (``window_mfma_ok``)."""
@@ -776,9 +873,9 @@ def window_attn(q, pool, block_tables, row_ent, pos, sink, scale: float, win: in
             k = kv[:, :G * D].view(-1, G, D).repeat_interleave(HG, 1)       # [n, H, D]
             v = kv[:, G * D:].view(-1, G, V).repeat_interleave(HG, 1)
             s = torch.einsum("hd,nhd->hn", q[r].float().view(H, D), k) * scale
-            m = torch.maximum(s.max(-1).values, sink)
+            m = s.max(-1).values if sink is None else torch.maximum(s.max(-1).values, sink)
             e = torch.exp(s - m[:, None])
-            den = e.sum(-1) + torch.exp(sink - m)
+            den = e.sum(-1) if sink is None else e.sum(-1) + torch.exp(sink - m)
             out[r] = (torch.einsum("hn,nhv->hv", e / den[:, None], v).reshape(H * V) * out_scale).to(out.dtype)
         return out
     _rows2d(q, "q")
@@ -788,7 +885,8 @@ def window_attn(q, pool, block_tables, row_ent, pos, sink, scale: float, win: in
     assert pool.dim() == 2 and pool.is_contiguous() and pool.shape[1] == G * (D + V)
     assert block_tables.dtype == torch.int32 and block_tables.is_contiguous()
     assert row_ent.dtype == torch.int32 and pos.dtype == torch.int32
-    _vec(sink, H, "sink")
+    if sink is not None:
+        _vec(sink, H, "sink")
     if win < 1:
         raise ValueError("window of %d keys" % win)
     if units is not None and window_mfma_ok(q, pool, D, V):
@@ -808,13 +906,13 @@ def window_attn(q, pool, block_tables, row_ent, pos, sink, scale: float, win: in
         _chk(lib().p2p_sm_window_attn_mfma(q.data_ptr(), q.stride(0), pool.data_ptr(),
                                            block_tables.data_ptr(), block_tables.shape[1],
                                            row_ent.data_ptr(), pos.data_ptr(), units.data_ptr(), U,
-                                           sink.data_ptr(), scale, win, out.data_ptr(),
+                                           _lib.ptr(sink), scale, win, out.data_ptr(),
                                            out.stride(0), H, G, D, V, page, splits, _lib.ptr(part),
                                            out_scale, _st(q)), "window_attn_mfma")
         return out
     _chk(lib().p2p_sm_window_attn(q.data_ptr(), q.stride(0), pool.data_ptr(),
                                   block_tables.data_ptr(), block_tables.shape[1],
-                                  row_ent.data_ptr(), pos.data_ptr(), sink.data_ptr(), scale, win,
+                                  row_ent.data_ptr(), pos.data_ptr(), _lib.ptr(sink), scale, win,
                                   out.data_ptr(), out.stride(0), R, H, G, D, V, page, out_scale,
                                   _f32(q), _st(q)), "window_attn")
     return out
@@ -940,27 +1038,99 @@ def gated_delta_scan(conv, araw, braw, gate, A_log, dt_bias, normw, state, ent, 
     return out
 
 
+def mlstm_scan(proj, bi, bf, cap: float, normw, state, mstate, ent, ent_host, out, H: int, D: int,
+               V: int, eps: float, out_scale: float = 1.0):
+    """Matrix memory of the mLSTM.  proj = [q (H*D) | k (H*D) | v (H*V) | gate (H*V) | zi (H) |
+    zf (H)] raw projections of the step's rows.  Per head, with the capped log gates
+    i = cap tanh((zi + bi) / cap), f = logsigmoid(cap tanh((zf + bf) / cap)) and the running
+    maximum m <- max(f + m, i) (m = 0 before position 0):
+        S <- exp(f + m' - m) S + exp(i - m) k v^T,   n likewise with k alone,
+        o = S^T (q D^-1/2) / (max(|n . q D^-1/2|, exp(-m)) + 1e-6);
+    every head's o is RMS-normalised over V, weighted by normw [H*V] and multiplied by
+    sigmoid(gate).  state fp32 [slots, H, D, V + 1] (column V holds n), mstate fp32 [slots, H];
+    out [R, H*V] activation type.  Gates, maximum, exponentials and state are fp32."""
+    nq, nv = H * D, H * V
+    if not proj.is_cuda:
+        for row0, cnt, start, slot in ent_host:
+            S = state[slot] if start > 0 else torch.zeros_like(state[slot])
+            m = mstate[slot] if start > 0 else torch.zeros_like(mstate[slot])
+            for t in range(row0, row0 + cnt):
+                row = proj[t].float()
+                q = row[:nq].view(H, D) * D ** -0.5
+                k = row[nq:2 * nq].view(H, D)
+                v1 = torch.cat([row[2 * nq:2 * nq + nv].view(H, V), torch.ones(H, 1)], 1)
+                zi, zf = row[2 * nq + 2 * nv:2 * nq + 2 * nv + H], row[2 * nq + 2 * nv + H:2 * nq + 2 * nv + 2 * H]
+                i = cap * torch.tanh((zi + bi) / cap)
+                f = torch.nn.functional.logsigmoid(cap * torch.tanh((zf + bf) / cap))
+                mn = torch.maximum(f + m, i)
+                a, b = torch.exp(f + m - mn), torch.exp(i - mn)
+                S = a[:, None, None] * S + (b[:, None] * k)[:, :, None] * v1[:, None, :]
+                m = mn
+                o = torch.einsum("hdv,hd->hv", S, q)
+                den = torch.maximum(o[:, V].abs(), torch.exp(-m)) + 1e-6
+                o = _rms(o[:, :V] / den[:, None], eps).reshape(nv) * normw
+                o = o * torch.sigmoid(row[2 * nq + nv:2 * nq + 2 * nv]) * out_scale
+                out[t] = o.to(out.dtype)
+            state[slot] = S
+            mstate[slot] = m
+        return out
+    _rows2d(proj, "proj")
+    _rows2d(out, "out")
+    assert proj.shape[1] >= 2 * nq + 2 * nv + 2 * H and out.shape[1] == nv and out.dtype == proj.dtype
+    _vec(bi, H, "bi")
+    _vec(bf, H, "bf")
+    _vec(normw, nv, "normw")
+    assert state.dtype == torch.float32 and state.is_contiguous() and state.shape[1:] == (H, D, V + 1)
+    assert mstate.dtype == torch.float32 and mstate.is_contiguous() and mstate.shape[1:] == (H,)
+    assert mstate.shape[0] == state.shape[0]
+    assert ent.dtype == torch.int32 and ent.is_contiguous() and ent.shape[1] == 4
+    if D > 256 or V > 255:
+        raise ValueError("mlstm_scan: key %d / value %d sizes above 256 / 255" % (D, V))
+    R = out.shape[0]
+    coef = torch.empty(R, H, 3, device=proj.device, dtype=torch.float32)
+    vent = cent = cs = cd = None
+    NV = 0
+    if _chunked(ent_host):
+        vent, cent = (t_.to(proj.device) for t_ in scan_chunks(ent_host, SCAN_CHUNK))
+        NV = vent.shape[0]
+        cs = torch.empty(NV, H, D, V + 1, device=proj.device, dtype=torch.float32)
+        cd = torch.empty(NV, H, D, device=proj.device, dtype=torch.float32)
+    _chk(lib().p2p_sm_mlstm_scan(proj.data_ptr(), proj.stride(0), bi.data_ptr(), bf.data_ptr(), cap,
+                                 normw.data_ptr(), state.data_ptr(), mstate.data_ptr(),
+                                 coef.data_ptr(), ent.data_ptr(), ent.shape[0], _lib.ptr(cs),
+                                 _lib.ptr(cd), _lib.ptr(vent), NV, _lib.ptr(cent), out.data_ptr(),
+                                 out.stride(0), H, D, V, eps, out_scale, _f32(proj), _st(proj)),
+         "mlstm_scan")
+    return out
+
+
 # ------------------------------------------------------------------ mixture of experts
-def group_route(h, wr, top: int, groups: int, keep: int, ids, wts, cnt, rows):
-    """Sigmoid router with group-limited choice.  z = h wr^T in fp32 (wr fp32 [E, W]),
-    s = sigmoid(z); the E experts are cut into ``groups`` contiguous blocks of equal size, a
-    block is ranked by its top-2 sum of s, experts outside the ``keep`` best blocks are
-    struck out; the
-    ``top`` largest s among them win (ties: the lower index), their weights are their s.
+def group_route(h, wr, top: int, groups: int, keep: int, ids, wts, cnt, rows,
+                score: str = "sigmoid", corr=None, group_score: str = "top2"):
+    """Router with group-limited choice.  z = h wr^T in fp32 (wr fp32 [E, W]); the scores are
+    s = sigmoid(z) or (``score`` "softmax") softmax(z) over all E; the choice is made on
+    c = s + corr (corr fp32 [E], optional).  The E experts are cut into ``groups`` contiguous
+    blocks of equal size, a block is ranked by the sum of its two best c (``group_score``
+    "top2") or by its best c ("max"), experts outside the ``keep`` best blocks are struck out;
+    the ``top`` largest c among the rest win (ties: the lower index), their weights are their s.
     ids int32 / wts fp32 [R, top]; cnt int32 [E] and rows int32 [E, R*top] list per expert the
     slots (row * top + k) routed to it (cnt is cleared here)."""
     R = h.shape[0]
     E = wr.shape[0]
     per = E // groups
+    if score not in ("sigmoid", "softmax") or group_score not in ("top2", "max"):
+        raise ValueError("group_route: score %r / group score %r" % (score, group_score))
     if not h.is_cuda:
-        s = torch.sigmoid(h.float() @ wr.t())                                     # [R, E]
-        gs = s.view(R, groups, per).topk(min(2, per), dim=-1).values.sum(-1)      # [R, groups]
+        z = h[:R].float() @ wr.t()                                                # [R, E]
+        s = torch.sigmoid(z) if score == "sigmoid" else torch.softmax(z, -1)
+        c = s if corr is None else s + corr
+        gs = c.view(R, groups, per).topk(min(2, per) if group_score == "top2" else 1, dim=-1).values.sum(-1)
         best = gs.topk(keep, dim=-1).indices
         ok = torch.zeros(R, groups, dtype=torch.bool).scatter_(1, best, True)
-        masked = torch.where(ok.repeat_interleave(per, 1), s, torch.full_like(s, -1.0))
-        w, i = masked.topk(top, dim=-1)
+        masked = torch.where(ok.repeat_interleave(per, 1), c, torch.full_like(c, -float("inf")))
+        i = masked.topk(top, dim=-1).indices
         ids[:R] = i.to(torch.int32)
-        wts[:R] = w
+        wts[:R] = s.gather(1, i)
         cnt.zero_()
         for slot, e in enumerate(i.reshape(-1).tolist()):
             rows[e, int(cnt[e])] = slot
@@ -971,6 +1141,8 @@ def group_route(h, wr, top: int, groups: int, keep: int, ids, wts, cnt, rows):
     assert E % groups == 0 and 1 <= keep <= groups and 1 <= top <= keep * per
     if E > 1024:
         raise ValueError("group_route: %d experts > 1024" % E)
+    if corr is not None:
+        _vec(corr, E, "corr")
     assert ids.dtype == torch.int32 and ids.is_contiguous() and ids.shape == (R, top)
     assert wts.dtype == torch.float32 and wts.is_contiguous() and wts.shape == (R, top)
     assert cnt.dtype == torch.int32 and cnt.numel() == E
@@ -978,8 +1150,10 @@ def group_route(h, wr, top: int, groups: int, keep: int, ids, wts, cnt, rows):
         and rows.shape[1] >= R * top
     cnt.zero_()
     _chk(lib().p2p_sm_group_route(h.data_ptr(), h.stride(0), wr.data_ptr(), R, h.shape[1], E, top,
-                                  groups, keep, ids.data_ptr(), wts.data_ptr(), cnt.data_ptr(),
-                                  rows.data_ptr(), rows.stride(0), _f32(h), _st(h)), "group_route")
+                                  groups, keep, 1 if score == "softmax" else 0, _lib.ptr(corr),
+                                  1 if group_score == "max" else 0, ids.data_ptr(),
+                                  wts.data_ptr(), cnt.data_ptr(), rows.data_ptr(), rows.stride(0),
+                                  _f32(h), _st(h)), "group_route")
     return ids, wts
 
 
@@ -995,7 +1169,7 @@ def interleave_gate_up(gate, up):
 
 
 def expert_gemm(x, x_div: int, w, cnt, rows, out, total_slots: int, act_limit=None,
-                act_alpha: float = 1.702):
+                act_alpha: float = 1.702, relu2: bool = False):
     """Per expert e and each of its routed slots s = rows[e, i] (i < cnt[e]):
     out[s] = x[s // x_div] @ w[e]^T.  w [E, N, K] (activation type), x [*, K], out [slots, N].
     total_slots: the slots over all experts (every slot is in exactly one list; the grid is
@@ -1003,9 +1177,14 @@ def expert_gemm(x, x_div: int, w, cnt, rows, out, total_slots: int, act_limit=No
     result does not depend on the other slots.
     act_limit: w = ``interleave_gate_up(gate, up)`` and out [slots, N/2] receives
     min(g, L) * sigmoid(alpha * min(g, L)) * (clamp(u, -L, L) + 1) of the two products (fp32
-    before the rounding) instead of the products themselves."""
+    before the rounding) instead of the products themselves.
+    relu2: out receives relu(.)^2 of every product (an ungated unit; fp32 before the rounding).
+    cnt may list more experts than w holds (experts without weights): their slots are left
+    out."""
     E, N, K = w.shape
     fused = act_limit is not None
+    if fused and relu2:
+        raise ValueError("expert_gemm: one activation at a time")
     if not x.is_cuda:
         for e in range(E):
             sl = rows[e, :int(cnt[e])].long()
@@ -1017,32 +1196,46 @@ def expert_gemm(x, x_div: int, w, cnt, rows, out, total_slots: int, act_limit=No
                 g = torch.clamp(y[:, :, 0], max=act_limit)
                 u = torch.clamp(y[:, :, 1], -act_limit, act_limit)
                 y = (g * torch.sigmoid(act_alpha * g) * (u + 1)).reshape(-1, N // 2)
+            elif relu2:
+                y = torch.relu(y) ** 2
             out[sl] = y.to(out.dtype)
         return out
     _rows2d(x, "x")
     _rows2d(out, "out")
     assert w.is_contiguous() and x.shape[1] == K and out.shape[1] == (N // 2 if fused else N)
-    assert x.dtype == w.dtype == out.dtype and cnt.numel() == E
+    assert x.dtype == w.dtype == out.dtype and cnt.numel() >= E
     if fused and N % 32:
         raise ValueError("fused expert activation needs gate / up widths that are multiples of 16")
     _chk(lib().p2p_sm_expert_gemm(x.data_ptr(), x.stride(0), x_div, w.data_ptr(), cnt.data_ptr(),
                                   rows.data_ptr(), rows.stride(0), out.data_ptr(), out.stride(0),
-                                  E, N, K, total_slots, 1 if fused else 0,
+                                  E, N, K, total_slots, 1 if fused else 2 if relu2 else 0,
                                   float(act_limit) if fused else 0.0, act_alpha, _f32(x), _st(x)),
          "expert_gemm")
     return out
 
 
-def expert_combine(y, wts, out):
-    """out[r] = sum_k wts[r, k] * y[r * top + k] (fp32 sum, activation-typed result)."""
+def expert_combine(y, wts, out, ids=None, n_real: int = 0, x=None):
+    """out[r] = sum_k wts[r, k] * y[r * top + k] (fp32 sum, activation-typed result).  With
+    ids (int32 [R, top]) a slot whose expert index is >= n_real stands for an expert that hands
+    its input back: its term is wts[r, k] * x[r]."""
     R, top = wts.shape
     if not y.is_cuda:
-        out[:R] = (y[:R * top].float().view(R, top, -1) * wts[:, :, None]).sum(1).to(out.dtype)
+        t = y[:R * top].float().view(R, top, -1)
+        if ids is not None:
+            t = torch.where((ids[:R] >= n_real)[:, :, None], x[:R].float()[:, None, :], t)
+        out[:R] = (t * wts[:, :, None]).sum(1).to(out.dtype)
         return out
     _rows2d(y, "y")
     _rows2d(out, "out")
     assert y.shape[0] >= R * top and out.shape[1] == y.shape[1] and y.dtype == out.dtype
+    ldx = 0
+    if ids is not None:
+        _rows2d(x, "x")
+        assert ids.dtype == torch.int32 and ids.is_contiguous() and ids.shape == (R, top)
+        assert x.shape[1] == y.shape[1] and x.shape[0] >= R and x.dtype == y.dtype
+        ldx = x.stride(0)
     _chk(lib().p2p_sm_expert_combine(y.data_ptr(), y.stride(0), wts.data_ptr(), out.data_ptr(),
-                                     out.stride(0), R, top, y.shape[1], _f32(y), _st(y)),
-         "expert_combine")
+                                     out.stride(0), R, top, y.shape[1], _lib.ptr(ids), n_real,
+                                     _lib.ptr(x if ids is not None else None), ldx, _f32(y),
+                                     _st(y)), "expert_combine")
     return out

@@ -114,6 +114,15 @@ def _hybrid_presets() -> dict:
                     "right": {"heads": 4, "kv_heads": 2, "dim": 32, "vdim": 64, "conv": 4},
                     "left_scale": 1.0, "right_scale": 1.0},
           "mlp": {"kind": "dense", "ff": 512}}
+    ml = {"type": "mlstm", "mixer": {"heads": 4, "dim": 32, "vdim": 64, "gate_cap": 15.0}, "mlp": None}
+    at = {"type": "attention",
+          "mixer": {"heads": 8, "kv_heads": 2, "dim": 32, "vdim": 32, "scale": 32 ** -0.5,
+                    "rot": {"base": 10000.0, "dims": 32,
+                            "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 512}}},
+          "mlp": None}
+    gelu = {"kind": "dense", "ff": 512}
+    smoe = {"kind": "moe", "expert": {"ff": 128}, "shared": {"ff": 256},
+            "router": {"experts": 6, "identity": 2, "top": 2, "groups": {"count": 4, "keep": 2}}}
     return {"tiny-regesun": HybridConfig.from_dict(
         {"architecture": "Regesun", "width": 256, "vocab": 512, "max_positions": 4096,
          "norm": {"eps": 1e-5}, "layers": [gd, mb, la, mb, gd, la], "eos_token_id": [2]},
@@ -121,12 +130,17 @@ def _hybrid_presets() -> dict:
         "tiny-rotutar": HybridConfig.from_dict(
         {"architecture": "Rotutar", "width": 256, "vocab": 512, "norm": {"eps": 1e-5, "groups": 4},
          "logit_softcap": 50.0, "layers": [hg, dict(hg, mlp=moe), pa, hg, dict(hg, mlp=moe), pa],
-         "eos_token_id": [2]}, name="tiny-rotutar")}
+         "eos_token_id": [2]}, name="tiny-rotutar"),
+        "tiny-futetar": HybridConfig.from_dict(
+        {"architecture": "Futetar", "width": 256, "vocab": 512, "norm": {"eps": 1e-6},
+         "layers": [dict(ml, mlp=gelu), dict(ml, mlp=smoe), dict(at, mlp=gelu),
+                    {"type": "attention", "mixer": dict(at["mixer"], kv_from=2), "mlp": smoe}],
+         "eos_token_id": [2]}, name="tiny-futetar")}
 
 
 def get_config(name: str):
     key = ALIASES.get(name, name)
-    if key not in PRESETS and key.endswith(("regesun", "rotutar")):
+    if key not in PRESETS and key.endswith(("regesun", "rotutar", "futetar")):
         hp = _hybrid_presets()
         if key in hp:
             return hp[key]

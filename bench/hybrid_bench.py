@@ -1,12 +1,13 @@
-"""Prefill and decode throughput of hybrid models (Regesun, Rotutar) at layer sizes that
+"""Prefill and decode throughput of hybrid models (Regesun, Rotutar, Futetar) at layer sizes that
 resemble real models, beside a dense Llama of the same width, depth and parameter count on
 the same engine entry point (``generate``).  Random weights, random tokens.
 
-    python bench.py --hybrid [--hybrid-design regesun|rotutar|both] [--hybrid-sizes 1024,2048]
+    python bench.py --hybrid [--hybrid-design regesun|rotutar|futetar|both] [--hybrid-sizes 1024,2048]
                     [--steps K] [--warmup W]
 
 ``--hybrid-design rotutar`` runs Rotutar beside Regesun (the closest model: same engine, same
-width and depth) instead of the Llama.
+width and depth) instead of the Llama; ``futetar`` runs Futetar beside Rotutar (gated scans,
+grouped-query attention and routed experts in both).
 
 One JSON line per (size, model): prefill tokens/s of one long prompt (``prompt`` tokens),
 decode tokens/s of ``batch`` sequences.  These lines are not the headline metric.
@@ -58,6 +59,30 @@ def rotutar_config(width: int):
         {"architecture": "Rotutar", "width": width, "vocab": 32000,
          "norm": {"eps": 1e-5, "groups": 4}, "logit_softcap": 50.0,
          "layers": [hg, dict(hg, mlp=moe), hg, pa] * 4}, name="rotutar-w%d" % width)
+
+
+def futetar_config(width: int):
+    """A Futetar stack at a given width: blocks of mlstm+dense ff / mlstm+moe / attention+dense ff /
+    attention on the previous layer's keys and values + moe, 128-wide heads."""
+    from p2p_llm_chat_go_amd.models.hybrid import HybridConfig
+
+    hd = 128
+    nh = width // hd
+    moe = {"kind": "moe", "expert": {"ff": width // 2}, "shared": {"ff": width // 2},
+           "router": {"experts": 8, "identity": 2, "top": 2, "groups": {"count": 5, "keep": 3}}}
+    dense = {"kind": "dense", "ff": 4 * width}
+    ml = {"heads": nh, "dim": hd, "vdim": hd, "gate_cap": 15.0}
+    at = {"heads": nh, "kv_heads": max(1, nh // 4), "dim": hd, "vdim": hd, "scale": hd ** -0.5,
+          "rot": {"base": 500000.0, "dims": hd,
+                  "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}}
+    layers = []
+    for b in range(4):
+        layers += [{"type": "mlstm", "mixer": ml, "mlp": dense}, {"type": "mlstm", "mixer": ml, "mlp": moe},
+                   {"type": "attention", "mixer": at, "mlp": dense},
+                   {"type": "attention", "mixer": dict(at, kv_from=4 * b + 2), "mlp": moe}]
+    return HybridConfig.from_dict(
+        {"architecture": "Futetar", "width": width, "vocab": 32000, "norm": {"eps": 1e-6},
+         "layers": layers}, name="futetar-w%d" % width)
 
 
 def n_params(cfg) -> int:
@@ -126,8 +151,9 @@ def run(a):
         hcfg = regesun_config(width)
         params = n_params(hcfg)
         lcfg = llama_like(width, hcfg.n_layers, params)
-        todo = {"regesun": (hcfg, lcfg), "rotutar": (rotutar_config(width), hcfg),
-                "both": (rotutar_config(width), hcfg, lcfg)}[design]
+        todo = {"regesun": lambda: (hcfg, lcfg), "rotutar": lambda: (rotutar_config(width), hcfg),
+                "futetar": lambda: (futetar_config(width), rotutar_config(width)),
+                "both": lambda: (rotutar_config(width), hcfg, lcfg)}[design]()
         for cfg in todo:
             if getattr(a, "hybrid_only", None) and a.hybrid_only not in cfg.name:
                 continue

@@ -94,17 +94,20 @@ window_attn_k(const T* __restrict__ q, int ldq, const T* __restrict__ pool,
               const int* __restrict__ bt, int max_pages, const int* __restrict__ row_ent,
               const int* __restrict__ pos, const float* __restrict__ sink, float scale, int win,
               T* __restrict__ out, int ldo, int H, int G, int D, int V, int page, int TK,
-              float out_scale) {
+              float out_scale, int HB) {
   extern __shared__ float smem[];
-  const int HG = H / G, g = blockIdx.y, h0 = g * HG;
+  // a block takes up to HB query heads of one key/value head (all of them when they fit)
+  const int nhb = (H / G + HB - 1) / HB;
+  const int g = blockIdx.y / nhb, hb0 = (blockIdx.y % nhb) * HB;
+  const int h0 = g * (H / G) + hb0, HG = min(HB, H / G - hb0);
   const int ldk = D + 1, ldv = V + 1, ldpool = G * (D + V);
-  float* sq = smem;                      // [HG][D]
-  float* sk = sq + HG * D;               // [TK][D + 1]
+  float* sq = smem;                      // [HB][D]
+  float* sk = sq + HB * D;               // [TK][D + 1]
   float* sv = sk + TK * ldk;             // [TK][V + 1]
-  float* sp = sv + TK * ldv;             // [HG][TK]
-  float* sm_ = sp + HG * TK;             // [HG] running max
-  float* sl = sm_ + HG;                  // [HG] running sum
-  float* sal = sl + HG;                  // [HG] rescale of this tile
+  float* sp = sv + TK * ldv;             // [HB][TK]
+  float* sm_ = sp + HB * TK;             // [HB] running max
+  float* sl = sm_ + HB;                  // [HB] running sum
+  float* sal = sl + HB;                  // [HB] rescale of this tile
   const int r = blockIdx.x, tid = threadIdx.x;
   const int p = pos[r];
   const int* pages = bt + (size_t)row_ent[r] * max_pages;
@@ -211,19 +214,23 @@ int p2p_sm_window_attn(const void* q, int ldq, const void* pool, const int* bt, 
                        float out_scale, int f32, hipStream_t st) {
   if (R <= 0) return 0;
   if (H < 1 || G < 1 || H % G || D < 1 || V < 1 || win < 1) return (int)hipErrorInvalidValue;
-  int HG = H / G, TK = WA_TK;
-  auto lds = [&](int tk) {
-    return ((size_t)HG * D + (size_t)tk * (D + 1) + (size_t)tk * (V + 1) + (size_t)HG * tk +
-            3 * HG) * 4;
+  int HG = H / G, TK = WA_TK, HB = HG;
+  auto lds = [&](int tk, int hb) {
+    return ((size_t)hb * D + (size_t)tk * (D + 1) + (size_t)tk * (V + 1) + (size_t)hb * tk +
+            3 * hb) * 4;
   };
-  while (TK > 2 && lds(TK) > 64 * 1024) TK /= 2;
-  if ((long)HG * V > (long)WA_ACC * WA_THREADS || HG > WA_THREADS || lds(TK) > 64 * 1024)
+  // heads per block: as many of the group as the accumulators and the LDS hold
+  while (HB > 1 && ((long)HB * V > (long)WA_ACC * WA_THREADS || HB > WA_THREADS ||
+                    lds(8, HB) > 64 * 1024))
+    HB = (HB + 1) / 2;
+  while (TK > 2 && lds(TK, HB) > 64 * 1024) TK /= 2;
+  if ((long)HB * V > (long)WA_ACC * WA_THREADS || lds(TK, HB) > 64 * 1024)
     return (int)hipErrorInvalidValue;
-  dim3 grid(R, G);
-  SM_DISPATCH_T(f32, hipLaunchKernelGGL(window_attn_k<T>, grid, dim3(WA_THREADS), lds(TK), st,
+  dim3 grid(R, G * ((HG + HB - 1) / HB));
+  SM_DISPATCH_T(f32, hipLaunchKernelGGL(window_attn_k<T>, grid, dim3(WA_THREADS), lds(TK, HB), st,
                                          (const T*)q, ldq, (const T*)pool, bt, max_pages, row_ent,
                                          pos, sink, scale, win, (T*)out, ldo, H, G, D, V, page, TK,
-                                         out_scale));
+                                         out_scale, HB));
   return (int)hipGetLastError();
 }
 

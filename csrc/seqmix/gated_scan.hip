@@ -13,9 +13,11 @@
 //   S <- a_t S + (b_t k) v^T,  n <- a_t n + b_t k,  o = S^T q / (max(|n . q|, exp(-m_t)) + 1e-6).
 // m_t depends on the gates alone, so a small kernel walks it first (mlstm_gates_k: a_t, b_t and
 // exp(-m_t) per token and head, the slot keeps m); with these coefficients the recurrence is
-// linear in (S, n) and runs here -- n is one more value column of the state, written with the
-// value 1, so n . q leaves the kernel as column V of S^T q.  The head's o is RMS-normalised,
-// weighted per channel of the head and gated by a sigmoid.
+// linear in (S, n) and runs here.  n is stored as one more value column of the state (column V
+// of V + 1) but not carried by the wavefronts that hold S: after a staged chunk's tokens have
+// gone through S, thread i walks n_i through the same tokens and leaves n_i q_i in place of q_i
+// in LDS, and the epilogue sums them per token.  The head's o is RMS-normalised, weighted per
+// channel of the head and gated by a sigmoid.
 //
 // The value columns of S are independent.  A wavefront covers 16 columns x 4 slices of the key
 // index; lane (c, s) keeps rows s*DQ .. s*DQ+DQ-1 of column c in registers (NC columns, 16
@@ -76,7 +78,9 @@ __global__ void __launch_bounds__(1024 / NC) gated_scan_k(ScanArgs a) {
   const Entry en = load_entry(a.ent, e);
   if (en.n <= 0) return;
   const bool trans = mode == 3;
-  const int NCOL = trans ? D : VS;             // columns of the matrix this block carries
+  const int NCOL = trans ? D : V;              // columns of the matrix the wavefronts carry
+  const int SST = trans ? D : VS;              // columns of a state row in memory
+  constexpr int NI = (DKP + 63) / 64;          // normaliser channels per thread at most
   const int nw = blockDim.x >> 6, VP = nw * WC;
   extern __shared__ __align__(16) float smem[];
   float* sq = smem;                  // [CT][DKP]
@@ -113,9 +117,15 @@ __global__ void __launch_bounds__(1024 / NC) gated_scan_k(ScanArgs a) {
     for (int q = 0; q < DQ; q++) {
       // loads at clamped addresses, selected afterwards, so that they go out together
       float v0 = (trans && i0 + q == j[c]) ? 1.0f : 0.0f;
-      float vv = from_state ? Sg[(size_t)min(i0 + q, D - 1) * NCOL + jc[c]] : v0;
+      float vv = from_state ? Sg[(size_t)min(i0 + q, D - 1) * SST + jc[c]] : v0;
       S[c][q] = (act[c] && i0 + q < D) ? vv : 0.0f;
     }
+  float nr[NI];   // matrix memory: the normaliser's channels threadIdx.x + k * blockDim.x
+#pragma unroll
+  for (int k = 0; k < NI; k++) {
+    int i = threadIdx.x + k * blockDim.x;
+    nr[k] = (MEM && from_state && i < D) ? Sg[(size_t)i * SST + V] : 0.0f;
+  }
   if (!DELTA && mode == 1)
     for (int i = threadIdx.x; i < DKP; i += blockDim.x) sP[i] = 1.0f;
   const float negA = DELTA ? -expf(a.A_log[h]) : 0.0f;
@@ -154,7 +164,6 @@ __global__ void __launch_bounds__(1024 / NC) gated_scan_k(ScanArgs a) {
         float vv = 0.0f;
         if (i < V) vv = DELTA ? a.conv[row * a.ldc + 2 * a.G * D + h * V + i]
                               : ldf(proj, row * a.ldp + 2 * H * D + h * V + i);
-        else if (MEM && i == V) vv = 1.0f;   // the normaliser's column
         sv[idx] = vv;
       }
     if (DELTA) {
@@ -248,11 +257,32 @@ __global__ void __launch_bounds__(1024 / NC) gated_scan_k(ScanArgs a) {
       }
     }
     __syncthreads();
+    if (MEM) {
+      // the normaliser through the chunk's tokens; n_i q_i replaces q_i for the epilogue
+#pragma unroll
+      for (int k = 0; k < NI; k++) {
+        int i = threadIdx.x + k * blockDim.x;
+        if (i < D) {
+          float n = nr[k];
+          for (int t = 0; t < ct; t++) {
+            n = sg[t * DKP + i] * n + sk[t * DKP + i];
+            if (mode != 1) sq[t * DKP + i] *= n;
+          }
+          nr[k] = n;
+        }
+      }
+      __syncthreads();
+    }
     if (mode == 0 || mode == 2)
     for (int t = wave; t < ct; t += nw) {
       size_t row = (size_t)(en.row0 + t0 + t);
       float den = 1.0f;
-      if (MEM) den = fmaxf(fabsf(so[t * VP + V]), a.coef[(row * H + h) * 3 + 2]) + 1e-6f;
+      if (MEM) {
+        float nq = 0.0f;
+        for (int i = lane; i < D; i += 64) nq += sq[t * DKP + i];
+        nq = wave_sum(nq);
+        den = fmaxf(fabsf(nq), a.coef[(row * H + h) * 3 + 2]) + 1e-6f;
+      }
       float ss = 0.0f;
       for (int i = lane; i < V; i += 64) {
         float o = MEM ? so[t * VP + i] / den : so[t * VP + i];
@@ -274,7 +304,8 @@ __global__ void __launch_bounds__(1024 / NC) gated_scan_k(ScanArgs a) {
     }
     // the next staging writes sq .. sb, whose readers passed the barrier above; `so` is
     // written again only after the next staging barrier, which every wave reaches after its
-    // share of this chunk's outputs
+    // share of this chunk's outputs (the matrix memory's epilogue reads sq as well)
+    if (MEM) __syncthreads();
   }
   if (mode != 2) {
 #pragma unroll
@@ -282,8 +313,15 @@ __global__ void __launch_bounds__(1024 / NC) gated_scan_k(ScanArgs a) {
       if (act[c]) {
 #pragma unroll
         for (int q = 0; q < DQ; q++)
-          if (i0 + q < D) Sg[(size_t)(i0 + q) * NCOL + j[c]] = S[c][q];
+          if (i0 + q < D) Sg[(size_t)(i0 + q) * SST + j[c]] = S[c][q];
       }
+    if (MEM) {
+#pragma unroll
+      for (int k = 0; k < NI; k++) {
+        int i = threadIdx.x + k * blockDim.x;
+        if (i < D) Sg[(size_t)i * SST + V] = nr[k];
+      }
+    }
   }
   if (!DELTA && mode == 1) {
     __syncthreads();
@@ -368,64 +406,87 @@ dense_chain_k(float* __restrict__ cs, const float* __restrict__ trans, float* __
     for (int i = rg; i < D; i += DC_RG) sg[(size_t)i * V + j] = scur[i * LD + col];
 }
 
-// Log gates of the matrix memory and their running maximum, one wavefront per (portion, head):
+// Log gates of the matrix memory and their running maximum, one block per (portion, head):
 //   i_t = cap tanh((zi_t + bi) / cap),  f_t = logsigmoid(cap tanh((zf_t + bf) / cap)),
 //   m_t = max(f_t + m_(t-1), i_t)  (m = 0 before position 0; the slot keeps it between steps),
 //   coef[t] = (exp(f_t + m_(t-1) - m_t), exp(i_t - m_t), exp(-m_t)).
-// The gates of 64 tokens are evaluated side by side, lane 0 walks the maximum through them.
+// A token is the map m -> max(F + m, I) with (F, I) = (f_t, i_t); maps compose as
+// (F2, I2) o (F1, I1) = (F1 + F2, max(I1 + F2, I2)).  Every wavefront takes 64 tokens: an
+// inclusive scan of the maps by lane shuffles, the 64-token composite to LDS; one lane walks
+// m through the composites of the block's wavefronts; then every lane applies its prefix map
+// to the m at its group's start.  Any rounding of m only moves the scale on which S and n are
+// kept: the coefficients are formed from the same m values, so S e^m and n e^m stay exact.
 __device__ __forceinline__ float logsigmoidf_(float x) {
   return fminf(x, 0.0f) - log1pf(expf(-fabsf(x)));
 }
 
 template <typename T>
-__global__ void __launch_bounds__(64)
+__global__ void __launch_bounds__(1024)
 mlstm_gates_k(const T* __restrict__ proj, int ldp, int off_i, int off_f,
               const float* __restrict__ bi, const float* __restrict__ bf, float cap,
               float* __restrict__ mstate, const int* __restrict__ ent, float* __restrict__ coef,
               int H) {
-  __shared__ float si[64], sf[64], sm_[65];
-  const int e = blockIdx.x / H, h = blockIdx.x % H, lane = threadIdx.x;
+  __shared__ float cF[16], cI[16], cM[17];
+  const int e = blockIdx.x / H, h = blockIdx.x % H;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
   const Entry en = load_entry(ent, e);
   if (en.n <= 0) return;
   float* mg = mstate + (size_t)en.slot * H + h;
-  float m = en.start > 0 ? *mg : 0.0f;
-  for (int t0 = 0; t0 < en.n; t0 += 64) {
-    const int ct = min(64, en.n - t0);
-    const size_t row = (size_t)(en.row0 + t0 + min(lane, ct - 1));
-    float it = cap * tanhf((ldf(proj, row * ldp + off_i + h) + bi[h]) / cap);
-    float ft = logsigmoidf_(cap * tanhf((ldf(proj, row * ldp + off_f + h) + bf[h]) / cap));
-    si[lane] = it;
-    sf[lane] = ft;
-    __syncthreads();
-    if (lane == 0) {
-      float mm = m;
-      sm_[0] = mm;
-      for (int j = 0; j < ct; j++) {
-        mm = fmaxf(sf[j] + mm, si[j]);
-        sm_[j + 1] = mm;
+  float m0 = en.start > 0 ? *mg : 0.0f;
+  const float bih = bi[h], bfh = bf[h];
+  for (int t0 = 0; t0 < en.n; t0 += 64 * nw) {
+    const int t = t0 + wave * 64 + lane;
+    const bool ok = t < en.n;
+    const size_t row = (size_t)(en.row0 + min(t, en.n - 1));
+    float it = cap * tanhf((ldf(proj, row * ldp + off_i + h) + bih) / cap);
+    float ft = logsigmoidf_(cap * tanhf((ldf(proj, row * ldp + off_f + h) + bfh) / cap));
+    // tokens beyond the portion are the identity map
+    float F = ok ? ft : 0.0f, I = ok ? it : -INFINITY;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      float Fp = __shfl_up(F, o, 64), Ip = __shfl_up(I, o, 64);
+      if (lane >= o) {
+        I = fmaxf(Ip + F, I);
+        F = Fp + F;
       }
     }
+    if (lane == 63) {
+      cF[wave] = F;
+      cI[wave] = I;
+    }
     __syncthreads();
-    if (lane < ct) {
-      float mp = sm_[lane], mn = sm_[lane + 1];
+    if (threadIdx.x == 0) {
+      float mm = m0;
+      for (int w = 0; w < nw; w++) {
+        cM[w] = mm;
+        mm = fmaxf(cF[w] + mm, cI[w]);
+      }
+      cM[nw] = mm;
+    }
+    __syncthreads();
+    const float ms = cM[wave];              // m before this wavefront's first token
+    float mn = fmaxf(F + ms, I);            // m_t
+    float mp = __shfl_up(mn, 1, 64);        // m_(t-1)
+    if (lane == 0) mp = ms;
+    if (ok) {
       float* cf = coef + (row * H + h) * 3;
       cf[0] = expf(ft + mp - mn);
       cf[1] = expf(it - mn);
       cf[2] = expf(-mn);
     }
-    m = sm_[ct];
+    m0 = cM[nw];
     __syncthreads();
   }
-  if (lane == 0) *mg = m;
+  if (threadIdx.x == 0) *mg = m0;
 }
 
 template <int KIND>
 static int launch_scan(ScanArgs a, int E, int f32, hipStream_t st) {
   if (E <= 0) return 0;
   if (KIND != 2) a.VS = a.V;
-  if (a.H < 1 || a.D < 1 || a.V < 1 || a.D > 256 || a.VS > 256 || a.G < 1 || a.H % a.G)
+  if (a.H < 1 || a.D < 1 || a.V < 1 || a.D > 256 || a.V > 256 || a.G < 1 || a.H % a.G)
     return (int)hipErrorInvalidValue;
-  int cols = a.mode == 3 ? a.D : a.VS;
+  int cols = a.mode == 3 ? a.D : a.V;
   int dq = a.D <= 32 ? 8 : a.D <= 64 ? 16 : a.D <= 128 ? 32 : 64;
   // one column per lane: two (NC = 2) halve the wavefronts that read the staged vectors from
   // LDS but measured no faster (120 us against 110 us per 64-token pass at 128 x 128 states)
@@ -529,17 +590,20 @@ int p2p_sm_gated_delta_scan_chunked(const float* conv, int ldc, const void* araw
 
 // Matrix memory: proj = [q (H*D) | k (H*D) | v (H*V) | gate (H*V) | zi (H) | zf (H)] in the
 // activation type; state fp32 [slots, H, D, V + 1] (column V: the normaliser), mstate fp32
-// [slots, H]; coef fp32 [rows, H, 3] scratch; normw fp32 [H*V].  With NV > 0 the portions run
+// [slots, H]; coef fp32 [rows, H, 3] scratch; normw fp32 [H*V]; max_n: rows of the longest
+// portion (sizes the gates' blocks).  With NV > 0 the portions run
 // as chunks (vent / cent / cs [NV, H, D, V+1] / cd [NV, H, D]), else in one pass over `ent`.
 int p2p_sm_mlstm_scan(const void* proj, int ldp, const float* bi, const float* bf, float cap,
                       const float* normw, float* state, float* mstate, float* coef,
                       const int* ent, int E, float* cs, float* cd, const int* vent, int NV,
                       const int* cent, void* out, int ldo, int H, int D, int V, float eps,
-                      float out_scale, int f32, hipStream_t st) {
+                      float out_scale, int max_n, int f32, hipStream_t st) {
   if (E <= 0) return 0;
-  if (H < 1 || D < 1 || V < 1 || D > 256 || V > 255 || cap <= 0.0f) return (int)hipErrorInvalidValue;
+  if (H < 1 || D < 1 || V < 1 || D > 256 || V > 256 || cap <= 0.0f) return (int)hipErrorInvalidValue;
   const int off_i = 2 * H * D + 2 * H * V, off_f = off_i + H;
-  SM_DISPATCH_T(f32, hipLaunchKernelGGL(mlstm_gates_k<T>, dim3(E * H), dim3(64), 0, st,
+  // wavefronts per (portion, head): one per 64 tokens of the longest portion, 16 at most
+  const int gw = max(1, min(16, (max_n + 63) / 64));
+  SM_DISPATCH_T(f32, hipLaunchKernelGGL(mlstm_gates_k<T>, dim3(E * H), dim3(64 * gw), 0, st,
                                          (const T*)proj, ldp, off_i, off_f, bi, bf, cap, mstate,
                                          ent, coef, H));
   int err = (int)hipGetLastError();

@@ -32,9 +32,10 @@ __global__ void ff_act_k(const T* __restrict__ gu, int ld, T* __restrict__ out, 
   stf(out, (size_t)r * ldo + c, g * sigmoidf_(alpha * g) * (u + 1.0f));
 }
 
-// tanh form of gelu: 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))
+// tanh form of gelu: 0.5 z (1 + tanh(y)), y = sqrt(2/pi) (z + 0.044715 z^3), evaluated as
+// z * sigmoid(2 y), which is the same function (1 + tanh(y) = 2 sigmoid(2 y))
 __device__ __forceinline__ float gelu_tanhf_(float z) {
-  return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+  return z * sigmoidf_(1.5957691216057308f * (z + 0.044715f * z * z * z));
 }
 
 // [gate | up] -> act(gate) * up; act: 0 silu, 1 gelu (tanh form)

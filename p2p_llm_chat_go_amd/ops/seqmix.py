@@ -75,7 +75,7 @@ _SIGS = {
     "p2p_sm_mlstm_scan": [c_void_p, c_int, c_void_p, c_void_p, c_float, c_void_p, c_void_p,
                           c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
                           c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_float, c_float,
-                          c_int, c_void_p],
+                          c_int, c_int, c_void_p],
     "p2p_sm_softcap": [c_void_p, c_int, c_void_p, c_int, c_int, c_float, c_int, c_void_p],
     "p2p_sm_embed_rows": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                           c_void_p],
@@ -1084,8 +1084,8 @@ def mlstm_scan(proj, bi, bf, cap: float, normw, state, mstate, ent, ent_host, ou
     assert mstate.dtype == torch.float32 and mstate.is_contiguous() and mstate.shape[1:] == (H,)
     assert mstate.shape[0] == state.shape[0]
     assert ent.dtype == torch.int32 and ent.is_contiguous() and ent.shape[1] == 4
-    if D > 256 or V > 255:
-        raise ValueError("mlstm_scan: key %d / value %d sizes above 256 / 255" % (D, V))
+    if D > 256 or V > 256:
+        raise ValueError("mlstm_scan: key %d / value %d sizes above 256" % (D, V))
     R = out.shape[0]
     coef = torch.empty(R, H, 3, device=proj.device, dtype=torch.float32)
     vent = cent = cs = cd = None
@@ -1099,7 +1099,8 @@ def mlstm_scan(proj, bi, bf, cap: float, normw, state, mstate, ent, ent_host, ou
                                  normw.data_ptr(), state.data_ptr(), mstate.data_ptr(),
                                  coef.data_ptr(), ent.data_ptr(), ent.shape[0], _lib.ptr(cs),
                                  _lib.ptr(cd), _lib.ptr(vent), NV, _lib.ptr(cent), out.data_ptr(),
-                                 out.stride(0), H, D, V, eps, out_scale, _f32(proj), _st(proj)),
+                                 out.stride(0), H, D, V, eps, out_scale,
+                                 max(e[1] for e in ent_host), _f32(proj), _st(proj)),
          "mlstm_scan")
     return out
 

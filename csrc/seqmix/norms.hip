@@ -146,17 +146,26 @@ __global__ void add_norm_k(float* __restrict__ x, const T* __restrict__ a, int l
   const T* br = b ? b + (size_t)r * ldb : nullptr;
   float* xr = x + (size_t)r * n;
   if (n <= NV * (int)blockDim.x) {
-    float xv[NV], wv[NV];
+    // every load goes out before the first store (a store to x in between would hold back
+    // the later loads of x)
+    float xv[NV], wv[NV], yv[NV];
     float s2 = 0.0f;
 #pragma unroll
     for (int k = 0; k < NV; k++) {
       int i = threadIdx.x + k * blockDim.x;
       bool ok = i < n;
-      float y = ok ? ldf(ar, i) : 0.0f;
-      if (br && ok) y += ldf(br, i);
-      wv[k] = (ok && w2) ? w2[i] : 0.0f;
-      xv[k] = ok ? xr[i] + y : 0.0f;
-      if (ok) xr[i] = xv[k];
+      int ic = ok ? i : 0;
+      float y = ldf(ar, ic);
+      if (br) y += ldf(br, ic);
+      yv[k] = ok ? y : 0.0f;
+      wv[k] = (ok && w2) ? w2[ic] : 0.0f;
+      xv[k] = ok ? xr[ic] : 0.0f;
+    }
+#pragma unroll
+    for (int k = 0; k < NV; k++) {
+      int i = threadIdx.x + k * blockDim.x;
+      xv[k] += yv[k];
+      if (i < n) xr[i] = xv[k];
       s2 += xv[k] * xv[k];
     }
     if (!w2) return;

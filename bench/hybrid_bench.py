@@ -62,24 +62,24 @@ def rotutar_config(width: int):
 
 
 def futetar_config(width: int):
-    """A Futetar stack at a given width: blocks of mlstm+dense ff / mlstm+moe / attention+dense ff /
-    attention on the previous layer's keys and values + moe, 128-wide heads."""
+    """A Futetar stack at a given width: blocks of mlstm+dense ff / attention+moe / mlstm+moe /
+    attention on the block's first attention layer's keys and values + dense ff, 128-wide heads."""
     from p2p_llm_chat_go_amd.models.hybrid import HybridConfig
 
     hd = 128
     nh = width // hd
     moe = {"kind": "moe", "expert": {"ff": width // 2}, "shared": {"ff": width // 2},
-           "router": {"experts": 8, "identity": 2, "top": 2, "groups": {"count": 5, "keep": 3}}}
+           "router": {"experts": 8, "identity": 4, "top": 2, "groups": {"count": 4, "keep": 2}}}
     dense = {"kind": "dense", "ff": 4 * width}
-    ml = {"heads": nh, "dim": hd, "vdim": hd, "gate_cap": 15.0}
+    ml = {"heads": nh, "dim": hd, "vdim": hd, "gate_cap": 12.0}
     at = {"heads": nh, "kv_heads": max(1, nh // 4), "dim": hd, "vdim": hd, "scale": hd ** -0.5,
           "rot": {"base": 500000.0, "dims": hd,
                   "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}}
     layers = []
     for b in range(4):
-        layers += [{"type": "mlstm", "mixer": ml, "mlp": dense}, {"type": "mlstm", "mixer": ml, "mlp": moe},
-                   {"type": "attention", "mixer": at, "mlp": dense},
-                   {"type": "attention", "mixer": dict(at, kv_from=4 * b + 2), "mlp": moe}]
+        layers += [{"type": "mlstm", "mixer": ml, "mlp": dense}, {"type": "attention", "mixer": at, "mlp": moe},
+                   {"type": "mlstm", "mixer": ml, "mlp": moe},
+                   {"type": "attention", "mixer": dict(at, kv_from=4 * b + 1), "mlp": dense}]
     return HybridConfig.from_dict(
         {"architecture": "Futetar", "width": width, "vocab": 32000, "norm": {"eps": 1e-6},
          "layers": layers}, name="futetar-w%d" % width)

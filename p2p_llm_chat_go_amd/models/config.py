@@ -114,7 +114,7 @@ def _hybrid_presets() -> dict:
                     "right": {"heads": 4, "kv_heads": 2, "dim": 32, "vdim": 64, "conv": 4},
                     "left_scale": 1.0, "right_scale": 1.0},
           "mlp": {"kind": "dense", "ff": 512}}
-    ml = {"type": "mlstm", "mixer": {"heads": 4, "dim": 32, "vdim": 64, "gate_cap": 15.0}, "mlp": None}
+    ml = {"type": "mlstm", "mixer": {"heads": 4, "dim": 32, "vdim": 64, "gate_cap": 12.0}, "mlp": None}
     at = {"type": "attention",
           "mixer": {"heads": 8, "kv_heads": 2, "dim": 32, "vdim": 32, "scale": 32 ** -0.5,
                     "rot": {"base": 10000.0, "dims": 32,
@@ -133,8 +133,8 @@ def _hybrid_presets() -> dict:
          "eos_token_id": [2]}, name="tiny-rotutar"),
         "tiny-futetar": HybridConfig.from_dict(
         {"architecture": "Futetar", "width": 256, "vocab": 512, "norm": {"eps": 1e-6},
-         "layers": [dict(ml, mlp=gelu), dict(ml, mlp=smoe), dict(at, mlp=gelu),
-                    {"type": "attention", "mixer": dict(at["mixer"], kv_from=2), "mlp": smoe}],
+         "layers": [dict(at, mlp=gelu), dict(ml, mlp=smoe), dict(ml, mlp=gelu),
+                    {"type": "attention", "mixer": dict(at["mixer"], kv_from=0), "mlp": smoe}, ml],
          "eos_token_id": [2]}, name="tiny-futetar")}
 
 

@@ -305,6 +305,26 @@ def test_memory_far_tokens_and_long_decoding(dev, which):
     close(run_cuts(eng, "b", t2, [20] + [1] * (n - 20))[-1:], ref2[-1:])
 
 
+@pytest.mark.parametrize("dev", DEVICES)
+def test_scan_chunk_edges(dev):
+    """Long portions of a memory layer run as chunks of 64 tokens side by side once a portion
+    has 128 tokens: lengths just below, at and above these edges, alone and continued, with a
+    memory that keeps its first tokens."""
+    c, cfg, sd = make([layer(ML, None, heads=2, dim=16, vdim=16), layer(ML, DENSE)], seed=19)
+    for i in (0, 1):
+        sd["l%d.mix.f.b" % i] = torch.full_like(sd["l%d.mix.f.b" % i], 4.0)
+    t = toks(4 * PAGE + 2, cfg.vocab, 31)
+    ref = O.forward(c, sd, t)
+    eng = engine(cfg, sd, dev)
+    for cuts in ([127, 1, 128, 2], [128, 129], [129, 127, 2], [63, 65, 130], [191, 67], [192, 66], [193, 1, 64]):
+        close(run_cuts(eng, "a", t, cuts), ref)
+    # two long portions and a decoded token of other requests in one step
+    a, b = t[:200], t[:150]
+    eng.step([("x", a[:10], []), ("y", b[:149], [])])
+    out = eng.step([("x", a[10:], [189]), ("y", b[149:], [0]), ("z", t[:130], [129])])
+    close(out, torch.stack([ref[199], ref[149], ref[129]]))
+
+
 # ------------------------------------------------------------------ far keys, page borders, causal edge
 def spike_model(hot, qtok, beta=25.0, seed=11, borrowed=False):
     """Attention alone whose query projection is rebuilt so that every query points along the

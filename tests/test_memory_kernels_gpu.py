@@ -31,9 +31,10 @@ def _d(*ts):
 
 
 @pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("H,D,V", [(3, 20, 12), (4, 56, 24), (2, 40, 72), (1, 130, 200), (6, 8, 15), (1, 1, 1)])
+@pytest.mark.parametrize("H,D,V", [(3, 20, 12), (4, 56, 24), (2, 40, 72), (1, 130, 200), (6, 8, 15), (1, 1, 1),
+                                   (2, 32, 32), (1, 256, 256)])
 @pytest.mark.parametrize("lens", [[37, 1, 5], [200, 3, 131]], ids=["short", "chunked"])
-@pytest.mark.parametrize("cap", [15.0, 0.7])
+@pytest.mark.parametrize("cap", [20.0, 0.7])
 def test_mlstm_scan(dt, H, D, V, lens, cap):
     g = torch.Generator().manual_seed(3)
     nq, nv = H * D, H * V

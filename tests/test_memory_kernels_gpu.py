@@ -51,7 +51,9 @@ def test_mlstm_scan(dt, H, D, V, lens, cap):
         sm.mlstm_scan(proj, bi, bf, cap, normw, S1, m1, ent_t, ent, o1, H, D, V, 1e-5, out_scale=1.3)
         sm.mlstm_scan(proj.to(DEV), *_d(bi, bf), cap, normw.to(DEV), S2, m2, ent_t.to(DEV), ent, o2,
                       H, D, V, 1e-5, out_scale=1.3)
-        torch.testing.assert_close(o2.cpu().float(), o1.float(), **_tol(dt))
+        tol = _tol(dt)
+        tol["atol"] *= max(1, D // 64)     # sums over the key index in another order
+        torch.testing.assert_close(o2.cpu().float(), o1.float(), **tol)
         torch.testing.assert_close(S2.cpu(), S1, rtol=1e-4, atol=1e-5)
         torch.testing.assert_close(m2.cpu(), m1, rtol=1e-5, atol=1e-5)
 

@@ -40,10 +40,10 @@ limit) and ``moe`` (sigmoid router, choice limited to the best groups of experts
 "Regesun" stacks the first three mixers in the sandwich form with learned positions;
 "Rotutar" stacks ``parallel`` (window attention beside the gated delta rule) and ``hgrn2``
 layers in the gated post-norm form, without positions other than the rotation, and caps
-its logits with a tanh.  "Futetar" stacks ``mlstm`` and ``attention`` layers in the parallel form
-(norm weights stored around zero), with gelu-gated dense feed-forwards and mixtures of
-squared-relu experts behind a softmax router.  A checkpoint is a ``config.json`` whose ``architecture`` names the
-design and one safetensors file (``load_dir``).
+its logits with a tanh.  "Futetar" stacks ``mlstm`` and ``attention`` layers in the parallel
+form (norm weights stored around zero), with gelu-gated dense feed-forwards and mixtures of
+squared-relu experts behind a softmax router.  A checkpoint is a ``config.json`` whose
+``architecture`` names the design and one safetensors file (``load_dir``).
 
 One ``forward`` serves every step: a flat list of token rows cut into entries (portions of
 prompts and single decoded tokens side by side, ``StepBatch``); attention layers read and

@@ -1,8 +1,10 @@
 """Sequence-mixer ops: recurrent state layers (generalized delta rule, Mamba-2, gated delta
-rule, HGRN2), latent attention and grouped-query attention with a sliding window and a
-softmax sink (query/key norm, rotary positions and the cache write in one pass), a
-group-limited expert router with grouped expert products, learned positions, and the norms
-and pointwise steps around them.
+rule, HGRN2, the mLSTM's matrix memory), latent attention and grouped-query attention with an
+optional sliding window and softmax sink (query/key norm over the row or per head, rotary
+positions on adjacent or half-split channel pairs and the cache write in one pass), a
+group-limited expert router (sigmoid or softmax scores, optional score correction) with
+grouped expert products and identity experts, learned positions, and the norms, residual
+passes and pointwise steps around them.
 
 GPU tensors always run the gfx950 kernels of ``csrc/seqmix`` (``libp2p_seqmix.so``, built on
 first use when missing); CPU tensors run the PyTorch rendering of the same math, which is

@@ -80,14 +80,22 @@ class Design:
     positions: str | None     # "learned": a position table is added to the embedding
     norm_offset: float = 0.0  # block and final norm weights are stored minus this (1: around zero)
     ff: tuple = ()            # (config kind, FEEDFORWARDS key) where the two differ
+    mixers: tuple = ()        # (config type, MIXERS key) where the two differ
+    scalar_norms: bool = False  # block and final norms have one weight for all channels
 
     def ff_key(self, kind: str) -> str:
         return dict(self.ff).get(kind, kind)
 
+    def mixer_key(self, kind: str) -> str:
+        return dict(self.mixers).get(kind, kind)
+
 
 DESIGNS = {"Regesun": Design("sandwich", "learned"), "Rotutar": Design("gated_post", None),
            "Futetar": Design("parallel", None, norm_offset=1.0,
-                             ff=(("dense", "dense_gelu"), ("moe", "moe_softmax")))}
+                             ff=(("dense", "dense_gelu"), ("moe", "moe_softmax"))),
+           "Tarunex": Design("parallel2", None, scalar_norms=True, ff=(("moe", "moe_top"),),
+                             mixers=(("latent_attention", "rope_latent_attention"),
+                                     ("attention", "biased_attention")))}
 NO_POS_LIMIT = 1 << 30
 
 
@@ -105,10 +113,26 @@ class HybridConfig:
     design: str = "Regesun"
     norm_groups: int = 1
     logit_softcap: float = 0.0
+    logit_scale: float = 1.0
+    embed_scale: float = 1.0
+    loop: tuple | None = None   # (start, stop, times): layers start .. stop-1 run `times` passes
 
     @property
     def traits(self) -> Design:
         return DESIGNS[self.design]
+
+    def runs(self) -> list:
+        """The layers in the order they run: (layer, pass, first of its pass) per layer run; a
+        layer outside the repeated stretch has pass None.  Every run has a cache of its own,
+        addressed by its place in this list."""
+        n = len(self.layers)
+        if not self.loop:
+            return [(i, None, False) for i in range(n)]
+        a, b, times = self.loop
+        runs = [(i, None, False) for i in range(a)]
+        for t in range(times):
+            runs += [(i, t, i == a) for i in range(a, b)]
+        return runs + [(i, None, False) for i in range(b, n)]
 
     @property
     def n_layers(self) -> int:
@@ -126,7 +150,7 @@ class HybridConfig:
         if design not in DESIGNS:
             raise KeyError("unknown design %r (known: %s)" % (design, ", ".join(sorted(DESIGNS))))
         for L in layers:
-            if L.kind not in MIXERS:
+            if DESIGNS[design].mixer_key(L.kind) not in MIXERS:
                 raise KeyError("unknown mixer %r (known: %s)" % (L.kind, ", ".join(sorted(MIXERS))))
             if L.mlp is not None and DESIGNS[design].ff_key(L.mlp.get("kind", "dense")) not in FEEDFORWARDS:
                 raise KeyError("unknown feed-forward kind %r" % L.mlp.get("kind"))
@@ -137,11 +161,21 @@ class HybridConfig:
             raise ValueError("width %d does not split into %d norm groups" % (width, groups))
         max_pos = int(c["max_positions"]) if DESIGNS[design].positions else \
             int(c.get("max_positions", NO_POS_LIMIT))
+        loop = None
+        if c.get("loop"):
+            loop = (int(c["loop"]["start"]), int(c["loop"]["stop"]), int(c["loop"]["times"]))
+            if not 0 <= loop[0] < loop[1] <= len(layers) or loop[2] < 1:
+                raise ValueError("loop over layers %d .. %d, %d times, of %d layers"
+                                 % (loop[0], loop[1] - 1, loop[2], len(layers)))
+            if DESIGNS[design].block != "parallel2":
+                raise ValueError("design %s does not repeat layers" % design)
         return cls(name=name or design.lower(), width=width,
                    vocab=int(c["vocab"]), layers=layers, eps=float(c["norm"]["eps"]),
                    max_pos=max_pos, bos_id=int(c.get("bos_token_id", 1)),
                    eos_ids=eos, design=design, norm_groups=groups,
                    logit_softcap=float(c.get("logit_softcap") or 0.0),
+                   logit_scale=float(c.get("logit_scale", 1.0)),
+                   embed_scale=float((c.get("embedding") or {}).get("scale", 1.0)), loop=loop,
                    is_moe=any(L.mlp is not None and L.mlp.get("kind") == "moe" for L in layers))
 
     def resolve(self, shapes: dict) -> "HybridConfig":
@@ -149,7 +183,7 @@ class HybridConfig:
         low-rank projections).  shapes: tensor name -> shape."""
         layers = []
         for i, L in enumerate(self.layers):
-            mx = MIXERS[L.kind].resolve_spec(dict(L.mixer), "l%d.mix." % i, shapes)
+            mx = MIXERS[self.traits.mixer_key(L.kind)].resolve_spec(dict(L.mixer), "l%d.mix." % i, shapes)
             layers.append(LayerSpec(L.kind, mx, L.mlp))
         return dataclasses.replace(self, layers=tuple(layers))
 
@@ -161,6 +195,12 @@ class HybridConfig:
             d["max_positions"] = self.max_pos
         if self.logit_softcap:
             d["logit_softcap"] = self.logit_softcap
+        if self.logit_scale != 1.0:
+            d["logit_scale"] = self.logit_scale
+        if self.embed_scale != 1.0:
+            d["embedding"] = {"scale": self.embed_scale}
+        if self.loop:
+            d["loop"] = dict(zip(("start", "stop", "times"), self.loop))
         return d
 
 
@@ -273,6 +313,7 @@ class Mixer:
     # that whoever owns the input (a layer with a gate, a ``parallel`` mixer) can run every
     # projection of the same input as one matrix product.
     w_in = None
+    b_in = None   # bias of the input product (activation type), or None
     wo = None
     n_mid = 0
 
@@ -285,7 +326,7 @@ class Mixer:
         return F.linear(self.mix(proj, b, cache, layer, mid), self.wo)
 
     def forward(self, h, b: "StepBatch", cache, layer: int):
-        return self.forward_proj(F.linear(h, self.w_in), b, cache, layer)
+        return self.forward_proj(F.linear(h, self.w_in, self.b_in), b, cache, layer)
 
 
 class GeneralDelta(Mixer):
@@ -498,6 +539,143 @@ class Attention(WindowAttention):
     PER_HEAD, HALF, SINK = True, True, False
 
 
+class BiasedAttention(Mixer):
+    """Causal grouped-query attention without rotation (``ops.seqmix.window_attn``): biased
+    q / k / v projections; the query is multiplied by a temperature that grows with the
+    logarithm of its position in steps of ``q_temp.every`` positions; scores are capped by
+    ``softcap * tanh(. / softcap)`` and lose ``r1_h * ln(1 + r2_h * distance)`` per head; the
+    softmax denominator holds one more 1 (a sink with score 0 and no value); every head leaves
+    multiplied by one sigmoid gate.  ``mask`` (a window) stays optional."""
+    kind = "biased_attention"
+
+    def _dims(self):
+        s = self.spec
+        self.H, self.D, self.V = int(s["heads"]), int(s["dim"]), int(s["vdim"])
+        self.G = int(s.get("kv_heads", self.H))
+        self.win = int(s["mask"]["size"]) if s.get("mask") else 1 << 30
+        self.scale = float(s["scale"]) if "scale" in s else self.D ** -0.5
+        self.cap = float(s.get("softcap") or 0.0)
+        qt = s.get("q_temp") or {}
+        self.qt_coef, self.qt_every = float(qt.get("coef", 0.0)), int(qt.get("every", 1))
+        if self.H % self.G or self.qt_every < 1 or self.cap < 0:
+            raise ValueError("biased_attention: %d heads / %d kv heads / temperature every %d / cap %g"
+                             % (self.H, self.G, self.qt_every, self.cap))
+        self.n_mid = self.H * self.V
+
+    def tensor_shapes(self):
+        self._dims()
+        H, G, D, V, W = self.H, self.G, self.D, self.V, self.width
+        return {"q": (H * D, W), "q.b": (H * D,), "k": (G * D, W), "k.b": (G * D,),
+                "v": (G * V, W), "v.b": (G * V,), "r1": (H,), "r2": (H,), "g": (H, W),
+                "o": (W, H * V)}
+
+    def load(self, get, dtype, dev):
+        self._dims()
+        # one projection for everything that reads the layer input: q | k | v | head gates
+        self.w_in = torch.cat([get(k) for k in ("q", "k", "v", "g")], 0).to(dev, dtype).contiguous()
+        self.b_in = torch.cat([get("q.b"), get("k.b"), get("v.b"),
+                               torch.zeros(self.H, dtype=get("q.b").dtype)]).to(dev, dtype).contiguous()
+        self.r1, self.r2 = _vec(get("r1"), dev), _vec(get("r2"), dev)
+        self.sink = torch.zeros(self.H, device=dev, dtype=torch.float32)
+        self.wo = get("o").to(dev, dtype).contiguous()
+
+    def cache_spec(self):
+        return ("paged", self.G * (self.D + self.V))
+
+    def mix(self, proj, b, cache, layer, out, out_scale=1.0):
+        H, G, D, V = self.H, self.G, self.D, self.V
+        pool = cache.paged[layer]
+        nq, nkv = H * D, G * (D + V)
+        q = torch.empty(b.R, nq, device=proj.device, dtype=proj.dtype)
+        sm.qtemp_kv_store(proj, nq, nkv, self.qt_coef, self.qt_every, b.pos, b.cache_rows, pool, q)
+        units = b.units(sm.window_rows_per_wave(H // G)) if sm.window_mfma_ok(q, pool, D, V) else None
+        sm.window_attn(q, pool, b.block_tables, b.row_ent, b.pos, self.sink, self.scale, self.win,
+                       out, PAGE, H, G, D, V, units=units, max_keys=b.max_keys, out_scale=out_scale,
+                       softcap=self.cap, dist=(self.r1, self.r2), gate=proj[:, nq + nkv:])
+        return out
+
+
+class RopeLatentAttention(Mixer):
+    """Latent attention with a rotated key part (``ops.seqmix.latent_attn``): queries come
+    through a normed low-rank latent; every token caches its normed key/value latent c
+    (``kv_rank`` numbers) and one rotated key part of ``rot_dim`` channels that all heads share.
+    A head's score is q_plain . (W_uk c) + q_rot . k_rot; the first term is evaluated in latent
+    space, (W_uk^T q_plain) . c, so keys and values are never formed: the cached row [c | k_rot]
+    meets the query [W_uk^T q_plain | q_rot], and the attended latent leaves through W_uv.
+    Rotation turns the pairs (2i, 2i+1).  Plain causal softmax (``mask`` optional), one sigmoid
+    gate per head."""
+    kind = "rope_latent_attention"
+
+    def _dims(self):
+        s = self.spec
+        self.H, self.D, self.V = int(s["heads"]), int(s["dim"]), int(s["vdim"])
+        self.Rd, self.rank, self.qrank = int(s["rot_dim"]), int(s["kv_rank"]), int(s["q_rank"])
+        self.win = int(s["mask"]["size"]) if s.get("mask") else 1 << 30
+        self.scale = float(s["scale"]) if "scale" in s else (self.D + self.Rd) ** -0.5
+        rot = s.get("rot") or {"dims": self.Rd, "base": 10000.0}
+        self.rot_dims, self.rot_base = int(rot["dims"]), float(rot["base"])
+        if self.rot_dims % 2 or self.rot_dims > self.Rd:
+            raise ValueError("rope_latent_attention: %d rotated of %d channels" % (self.rot_dims, self.Rd))
+        self.n_mid = self.H * self.V
+
+    @staticmethod
+    def resolve_spec(spec, prefix, shapes):
+        if "q_rank" not in spec and prefix + "dq" in shapes:
+            spec["q_rank"] = int(tuple(shapes[prefix + "dq"])[0])
+        return spec
+
+    def tensor_shapes(self):
+        self._dims()
+        H, D, V, Rd, r, qr, W = self.H, self.D, self.V, self.Rd, self.rank, self.qrank, self.width
+        return {"dq": (qr, W), "dq.norm": (qr,), "uq": (H * (D + Rd), qr), "dkv": (r + Rd, W),
+                "dkv.norm": (r,), "uk": (H * D, r), "uv": (H * V, r), "g": (H, W), "o": (W, H * V)}
+
+    def load(self, get, dtype, dev):
+        self._dims()
+        H, D, V, r = self.H, self.D, self.V, self.rank
+        # one projection for everything that reads the layer input: query latent | key/value
+        # latent | rotated key part | head gates
+        self.w_in = torch.cat([get("dq"), get("dkv"), get("g")], 0).to(dev, dtype).contiguous()
+        self.qnorm, self.cnorm = _vec(get("dq.norm"), dev), _vec(get("dkv.norm"), dev)
+        self.uq = get("uq").to(dev, dtype).contiguous()
+        self.uk = get("uk").to(dev, dtype).view(H, D, r).contiguous()
+        self.uvt = get("uv").to(dev, dtype).view(H, V, r).transpose(1, 2).contiguous()
+        self.inv_freq = sm.rope_inv_freq(self.rot_base, self.rot_dims, dev)
+        self.wo = get("o").to(dev, dtype).contiguous()
+
+    def cache_spec(self):
+        return ("paged", self.rank + self.Rd)
+
+    def mix(self, proj, b, cache, layer, out, out_scale=1.0):
+        H, D, V, Rd, r, qr = self.H, self.D, self.V, self.Rd, self.rank, self.qrank
+        R, dev, dt = b.R, proj.device, proj.dtype
+        pool = cache.paged[layer]
+        cq = torch.empty(R, qr, device=dev, dtype=dt)
+        sm.rmsnorm(proj[:, :qr], self.qnorm, self.eps, cq)
+        q = F.linear(cq, self.uq)                                                  # [R, H*(D+Rd)]
+        sm.rmsnorm(proj[:, qr:qr + r], self.cnorm, self.eps, pool[:, :r], out_rows=b.cache_rows)
+        nrot2 = self.rot_dims
+        kr = proj[:, qr + r:qr + r + Rd]
+        sm.rope_rows(kr, 1, 0, self.inv_freq, b.pos, pool[:, r:], 0, out_rows=b.cache_rows)
+        if nrot2 < Rd:   # channels of the shared key part beyond the rotated ones pass unchanged
+            pool[b.cache_rows.long(), r + nrot2:] = kr[:, nrot2:]
+        qa = torch.empty(H, R, r + Rd, device=dev, dtype=dt)
+        q3 = q.view(R, H, D + Rd)
+        torch.bmm(q3[:, :, :D].transpose(0, 1), self.uk, out=qa[:, :, :r])
+        sm.rope_rows(q[:, D:], H, D + Rd, self.inv_freq, b.pos, qa[0, :, r:], qa.stride(0))
+        if nrot2 < Rd:
+            qa[:, :, r + nrot2:] = q3[:, :, D + nrot2:].transpose(0, 1)
+        ol = torch.empty_like(qa)
+        units = b.units(sm.latent_rows_per_wave(H)) if sm.latent_mfma_ok(qa, pool) else None
+        sm.latent_attn(qa, pool, b.block_tables, b.row_ent, b.pos, None, self.scale, self.win, ol,
+                       PAGE, units=units, max_keys=b.max_keys)
+        o = torch.bmm(ol[:, :, :r], self.uvt)                                      # [H, R, V]
+        sm.sigmoid_gate(o, proj[:, qr + r + Rd:], out, H, V, per_head=True)
+        if out_scale != 1.0:
+            out.mul_(out_scale)
+        return out
+
+
 class MLSTM(Mixer):
     """Matrix memory of the xLSTM (``ops.seqmix.mlstm_scan``): per head a D x V memory and a
     normaliser, written through an exponential input gate and decayed by a sigmoid forget gate
@@ -671,7 +849,7 @@ class Parallel(Mixer):
 
 
 MIXERS = {c.kind: c for c in (GeneralDelta, Mamba2, LatentAttention, WindowAttention, GatedDelta,
-                              HGRN2, Parallel, Attention, MLSTM)}
+                              HGRN2, Parallel, Attention, MLSTM, BiasedAttention, RopeLatentAttention)}
 
 
 class DenseFF:
@@ -859,7 +1037,82 @@ class SoftmaxMoEFF:
         return y
 
 
-FEEDFORWARDS = {"dense": DenseFF, "moe": MoEFF, "dense_gelu": GeluFF, "moe_softmax": SoftmaxMoEFF}
+class TopMoEFF:
+    """Mixture of silu-gated experts, W_down (silu(W_gate h) * W_up h), behind a router with a
+    bias: the ``top`` largest logits win and the weights are the softmax over the winners'
+    logits only (``ops.seqmix.group_route``, "top_softmax").  An optional shared expert of the
+    same form runs for every token; its products ride on the layer's input and output
+    products."""
+
+    def __init__(self, spec: dict, width: int):
+        self.spec, self.width = spec, width
+        r = spec["router"]
+        self.E, self.top = int(r["experts"]), int(r["top"])
+        self.F = int(spec["expert"]["ff"])
+        self.Fs = self.n_mid = int(spec["shared"]["ff"]) if spec.get("shared") else 0
+        if not 1 <= self.top <= self.E:
+            raise ValueError("moe: %d experts, %d chosen" % (self.E, self.top))
+
+    def tensor_shapes(self):
+        d = {"router": (self.E, self.width), "router.b": (self.E,)}
+        for e in range(self.E):
+            d.update({"e%d.gate" % e: (self.F, self.width), "e%d.up" % e: (self.F, self.width),
+                      "e%d.down" % e: (self.width, self.F)})
+        if self.Fs:
+            d.update({"shared.gate": (self.Fs, self.width), "shared.up": (self.Fs, self.width),
+                      "shared.down": (self.width, self.Fs)})
+        return d
+
+    def load(self, get, dtype, dev):
+        self.wr, self.br = get("router").to(dev).float().contiguous(), _vec(get("router.b"), dev)
+        gate = torch.stack([get("e%d.gate" % e) for e in range(self.E)])
+        up = torch.stack([get("e%d.up" % e) for e in range(self.E)])
+        # widths that are multiples of 16: gate and up rows interleaved, so that the first
+        # product's epilogue applies the activation (otherwise gate | up and a pointwise pass)
+        self.fused = self.F % 16 == 0
+        w_gu = sm.interleave_gate_up(gate, up) if self.fused else torch.cat([gate, up], 1)
+        self.w_gu = w_gu.to(dev, dtype).contiguous()
+        self.w_down = torch.stack([get("e%d.down" % e) for e in range(self.E)]).to(dev, dtype).contiguous()
+        self.w_in = self.w_out = None
+        if self.Fs:
+            self.w_in = torch.cat([get("shared.gate"), get("shared.up")], 0).to(dev, dtype).contiguous()
+            self.w_out = get("shared.down").to(dev, dtype).contiguous()
+
+    def routed(self, h):
+        R, top, dev = h.shape[0], self.top, h.device
+        ids = torch.empty(R, top, device=dev, dtype=torch.int32)
+        wts = torch.empty(R, top, device=dev, dtype=torch.float32)
+        cnt = torch.empty(self.E, device=dev, dtype=torch.int32)
+        rows = torch.empty(self.E, R * top, device=dev, dtype=torch.int32)
+        sm.group_route(h, self.wr, top, 1, 1, ids, wts, cnt, rows, score="top_softmax", bias=self.br)
+        act = torch.empty(R * top, self.F, device=dev, dtype=h.dtype)
+        if self.fused:
+            sm.expert_gemm(h, top, self.w_gu, cnt, rows, act, R * top, silu_glu=True)
+        else:
+            gu = torch.empty(R * top, 2 * self.F, device=dev, dtype=h.dtype)
+            sm.expert_gemm(h, top, self.w_gu, cnt, rows, gu, R * top)
+            sm.glu_act(gu, act, "silu")
+        y = torch.empty(R * top, self.width, device=dev, dtype=h.dtype)
+        sm.expert_gemm(act, 1, self.w_down, cnt, rows, y, R * top)
+        out = torch.empty(R, self.width, device=dev, dtype=h.dtype)
+        return sm.expert_combine(y, wts, out)
+
+    def fill(self, proj, h, mid):
+        if self.Fs:
+            sm.glu_act(proj, mid, "silu")
+        return self.routed(h)
+
+    def forward(self, h):
+        y = self.routed(h)
+        if self.Fs:
+            mid = torch.empty(h.shape[0], self.Fs, device=h.device, dtype=h.dtype)
+            sm.glu_act(F.linear(h, self.w_in), mid, "silu")
+            y = y + F.linear(mid, self.w_out)
+        return y
+
+
+FEEDFORWARDS = {"dense": DenseFF, "moe": MoEFF, "dense_gelu": GeluFF, "moe_softmax": SoftmaxMoEFF,
+                "moe_top": TopMoEFF}
 
 
 # ---------------------------------------------------------------------------- weights
@@ -867,7 +1120,7 @@ class HybridLayer:
     def __init__(self, spec: LayerSpec, cfg: HybridConfig):
         self.block = cfg.traits.block
         self.norm_offset = cfg.traits.norm_offset
-        self.mixer = MIXERS[spec.kind](spec.mixer, cfg.width, cfg.eps)
+        self.mixer = MIXERS[cfg.traits.mixer_key(spec.kind)](spec.mixer, cfg.width, cfg.eps)
         self.ff = FEEDFORWARDS[cfg.traits.ff_key(spec.mlp.get("kind", "dense"))](spec.mlp, cfg.width) \
             if spec.mlp is not None else None
         # parallel: the layer's input and output products (mixer and feed-forward together)
@@ -877,6 +1130,13 @@ class HybridLayer:
         self.w_in1 = self.w_in2 = self.rg1b = self.rg2b = None
 
     def tensor_shapes(self, W):
+        if self.block == "parallel2":
+            d = {"norm1": ()}
+            d.update({"mix." + k: s for k, s in self.mixer.tensor_shapes().items()})
+            if self.ff is not None:
+                d["norm2"] = ()
+                d.update({"mlp." + k: s for k, s in self.ff.tensor_shapes().items()})
+            return d
         if self.block == "parallel":
             d = {"norm1": (W,)}
             d.update({"mix." + k: s for k, s in self.mixer.tensor_shapes().items()})
@@ -897,6 +1157,19 @@ class HybridLayer:
         self.mixer.load(lambda k: sd[p + "mix." + k], dtype, dev)
         if self.ff is not None:
             self.ff.load(lambda k: sd[p + "mlp." + k], dtype, dev)
+        if self.block == "parallel2":
+            # the mixer and the feed-forward read the same rows through norms of their own, so
+            # each has its input product; their output products are one
+            if self.mixer.w_in is None or self.mixer.wo is None:
+                raise ValueError("mixer %r cannot share the layer's products" % self.mixer.kind)
+            self.norm1 = (_vec(sd[p + "norm1"], dev).reshape(1) + self.norm_offset).contiguous()
+            outs = [self.mixer.wo]
+            if self.ff is not None:
+                self.norm2 = (_vec(sd[p + "norm2"], dev).reshape(1) + self.norm_offset).contiguous()
+                if self.ff.n_mid:
+                    outs.append(self.ff.w_out)
+            self.w_out_all = torch.cat(outs, 1).contiguous() if len(outs) > 1 else outs[0]
+            return
         if self.block == "parallel":
             if self.mixer.w_in is None or self.mixer.wo is None:
                 raise ValueError("mixer %r cannot share the layer's products" % self.mixer.kind)
@@ -928,9 +1201,12 @@ class HybridLayer:
 def tensor_shapes(cfg: HybridConfig) -> dict:
     """name -> shape of every tensor of a checkpoint of this config."""
     W = cfg.width
-    d = {"embed": (cfg.vocab, W), "final.norm": (W,), "head": (cfg.vocab, W)}
+    d = {"embed": (cfg.vocab, W), "final.norm": () if cfg.traits.scalar_norms else (W,),
+         "head": (cfg.vocab, W)}
     if cfg.traits.positions:
         d["pos"] = (cfg.max_pos, W)
+    if cfg.loop:
+        d["loop.step"] = (cfg.loop[2], W)
     for i, spec in enumerate(cfg.layers):
         d.update({"l%d.%s" % (i, k): s for k, s in HybridLayer(spec, cfg).tensor_shapes(W).items()})
     return d
@@ -952,8 +1228,10 @@ class HybridWeights:
                 raise ValueError("tensor %r has shape %s, the config gives %s" % (k, tuple(sd[k].shape), s))
         self.embed = sd["embed"].to(dev, dtype).contiguous()
         self.pos = sd["pos"].to(dev, dtype).contiguous() if cfg.traits.positions else None
-        self.final_norm = (_vec(sd["final.norm"], dev) + cfg.traits.norm_offset).contiguous()
+        self.final_norm = (_vec(sd["final.norm"], dev) + cfg.traits.norm_offset).expand(cfg.width).contiguous() \
+            if cfg.traits.scalar_norms else (_vec(sd["final.norm"], dev) + cfg.traits.norm_offset).contiguous()
         self.head = sd["head"].to(dev, dtype).contiguous()
+        self.loop_step = _vec(sd["loop.step"], dev) if cfg.loop else None
         self.layers = []
         for i, spec in enumerate(cfg.layers):
             L = HybridLayer(spec, cfg)
@@ -966,7 +1244,8 @@ class HybridWeights:
         return cls(cfg, random_state_dict(cfg, seed), device, dtype)
 
     def cache_specs(self) -> list:
-        return [L.mixer.cache_spec() for L in self.layers]
+        """What every layer run keeps between steps (a repeated layer once per pass)."""
+        return [self.layers[i].mixer.cache_spec() for i, _t, _f in self.cfg.runs()]
 
 
 def check_shared_caches(mixers: list):
@@ -1003,6 +1282,10 @@ def random_state_dict(cfg: HybridConfig, seed: int = 0) -> dict:
             t = 0.5 + 0.1 * torch.randn(*s, generator=g)
         elif leaf.endswith("A_log"):
             t = torch.rand(*s, generator=g) * 1.5 - 1.0
+        elif leaf.endswith(("mix.r1", "mix.r2")):
+            t = torch.rand(*s, generator=g) * (2.0 if leaf.endswith("r1") else 0.3)
+        elif k == "loop.step":
+            t = torch.randn(*s, generator=g) * 0.5
         elif leaf.endswith(("dt_bias", "mix.D")):
             t = torch.randn(*s, generator=g) * 0.5
         else:
@@ -1040,6 +1323,8 @@ class HybridModel:
             return self._forward_gated_post(b, layer_out)
         if cfg.traits.block == "parallel":
             return self._forward_parallel(b, layer_out)
+        if cfg.traits.block == "parallel2":
+            return self._forward_parallel2(b, layer_out)
         x = torch.empty(b.R, cfg.width, device=self.device, dtype=torch.float32)
         sm.embed_pos(w.embed, w.pos, b.ids, b.pos, x)
         h = torch.empty(b.R, cfg.width, device=self.device, dtype=self.dtype)
@@ -1065,9 +1350,52 @@ class HybridModel:
         hn = torch.empty(b.n_out, cfg.width, device=self.device, dtype=self.dtype)
         sm.rmsnorm(x, w.final_norm, cfg.eps, hn, parts=cfg.norm_groups, in_rows=b.out_rows)
         y = F.linear(hn, w.head)
-        if not cfg.logit_softcap:
+        if not cfg.logit_softcap and cfg.logit_scale == 1.0:
             return y.float()
-        return sm.softcap(y, cfg.logit_softcap, torch.empty(y.shape, device=y.device, dtype=torch.float32))
+        return sm.softcap(y, cfg.logit_softcap, torch.empty(y.shape, device=y.device, dtype=torch.float32),
+                          scale=cfg.logit_scale)
+
+    def _forward_parallel2(self, b: StepBatch, layer_out=None):
+        """x <- x + mixer(N(x) g1) + ff(N(x) g2) over the layer runs of the config (a stretch of
+        layers may run several passes; every run has its own cache).  One pass over the fp32
+        rows adds what the previous layer produced (or, at the start of a pass, the embedding
+        output and the pass's step vector) and writes both normed inputs of the next layer;
+        the mixer and the shared expert write the inputs of their output projections side by
+        side, one product sums the two in its fp32 accumulator, and the routed experts' sum is
+        added in the same residual pass."""
+        cfg, w = self.cfg, self.w
+        R, W = b.R, cfg.width
+        x = torch.empty(R, W, device=self.device, dtype=torch.float32)
+        sm.embed_rows(w.embed, b.ids, x, None, scale=cfg.embed_scale)
+        x0 = x.clone() if cfg.loop and cfg.loop[2] > 1 else None
+        h1 = torch.empty(R, W, device=self.device, dtype=self.dtype)
+        h2 = torch.empty(R, W, device=self.device, dtype=self.dtype)
+        runs = cfg.runs()
+        y = extra = None   # what the previous layer adds to x
+        for k, (i, t, first) in enumerate(runs):
+            L = w.layers[i]
+            n2, o2 = (L.norm2, h2) if L.ff is not None else (None, None)
+            if layer_out is not None and y is not None:   # the rows between two layers are asked for
+                sm.add_norm2(x, y, extra)
+                layer_out.append(x.clone())
+                y = extra = None
+            sm.add_norm2(x, y, extra, rows=x0 if first and t > 0 else None,
+                         vec=w.loop_step[t] if first else None, eps=cfg.eps,
+                         w1=L.norm1, out1=h1, w2=n2, out2=o2)
+            mm = L.mixer.n_mid
+            mid = torch.empty(R, L.w_out_all.shape[1], device=self.device, dtype=self.dtype)
+            L.mixer.mix(F.linear(h1, L.mixer.w_in, L.mixer.b_in), b, self.cache, k, mid[:, :mm])
+            extra = None
+            if L.ff is not None:
+                proj = F.linear(h2, L.ff.w_in) if L.ff.w_in is not None else None
+                extra = L.ff.fill(proj, h2, mid[:, mm:])
+            y = F.linear(mid, L.w_out_all)
+        sm.add_norm2(x, y, extra)
+        if layer_out is not None:
+            layer_out.append(x.clone())
+        if b.n_out == 0:
+            return None
+        return self._logits(x, b)
 
     def _forward_gated_post(self, b: StepBatch, layer_out=None):
         """x <- x + N(f(x) * sigmoid(R x + b)) per sublayer: the sublayer and its gate read the

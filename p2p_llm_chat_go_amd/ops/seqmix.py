@@ -64,7 +64,7 @@ _SIGS = {
                                 c_long, c_long, c_int, c_int, c_int, c_int, c_void_p, c_void_p],
     "p2p_sm_tanh": [c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "p2p_sm_sigmoid_gate": [c_void_p, c_long, c_long, c_void_p, c_int, c_void_p, c_int, c_int,
-                            c_int, c_int, c_int, c_void_p],
+                            c_int, c_int, c_int, c_int, c_void_p],
     "p2p_sm_ff_act": [c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_float, c_float, c_int,
                       c_void_p],
     "p2p_sm_gate_norm_add": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int,
@@ -74,22 +74,31 @@ _SIGS = {
                           c_void_p],
     "p2p_sm_add_norm": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_float,
                         c_void_p, c_void_p, c_int, c_int, c_void_p],
+    "p2p_sm_add_norm2": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int,
+                         c_int, c_float, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int,
+                         c_void_p, c_int, c_int, c_void_p],
+    "p2p_sm_rope_rows": [c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p,
+                         c_void_p, c_long, c_long, c_int, c_int, c_void_p],
+    "p2p_sm_qtemp_kv_store": [c_void_p, c_int, c_int, c_int, c_float, c_int, c_void_p, c_void_p,
+                              c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
     "p2p_sm_mlstm_scan": [c_void_p, c_int, c_void_p, c_void_p, c_float, c_void_p, c_void_p,
                           c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
                           c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_float, c_float,
                           c_int, c_int, c_void_p],
-    "p2p_sm_softcap": [c_void_p, c_int, c_void_p, c_int, c_int, c_float, c_int, c_void_p],
-    "p2p_sm_embed_rows": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
-                          c_void_p],
+    "p2p_sm_softcap": [c_void_p, c_int, c_void_p, c_int, c_int, c_float, c_float, c_int, c_void_p],
+    "p2p_sm_embed_rows": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float,
+                          c_int, c_void_p],
     "p2p_sm_qk_norm_rope_store": [c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p,
                                   c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_float,
                                   c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "p2p_sm_window_attn": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                            c_void_p, c_float, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int,
-                           c_int, c_int, c_float, c_int, c_void_p],
+                           c_int, c_int, c_float, c_float, c_void_p, c_void_p, c_void_p, c_int,
+                           c_int, c_void_p],
     "p2p_sm_window_attn_mfma": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                                 c_void_p, c_int, c_void_p, c_float, c_int, c_void_p, c_int, c_int,
-                                c_int, c_int, c_int, c_int, c_int, c_void_p, c_float, c_void_p],
+                                c_int, c_int, c_int, c_int, c_int, c_void_p, c_float, c_float,
+                                c_void_p, c_void_p, c_void_p, c_int, c_void_p],
     "p2p_sm_hgrn2_scan": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                           c_int, c_void_p, c_int, c_int, c_int, c_int, c_float, c_float, c_int,
                           c_void_p],
@@ -107,7 +116,7 @@ _SIGS = {
                                 c_int, c_void_p],
     "p2p_sm_group_route": [c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                            c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
-                           c_int, c_void_p],
+                           c_void_p, c_int, c_void_p],
     "p2p_sm_expert_gemm": [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                            c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_int,
                            c_void_p],
@@ -212,12 +221,12 @@ def embed_pos(embed, pos_table, ids, pos, out):
     return out
 
 
-def embed_rows(embed, ids, out, h_out=None):
-    """out[r] = embed[ids[r]] as fp32 rows; h_out (activation type, optional): the same rows
-    for a first sublayer that reads the residual stream as it is."""
+def embed_rows(embed, ids, out, h_out=None, scale: float = 1.0):
+    """out[r] = embed[ids[r]] * scale as fp32 rows; h_out (activation type, optional): the same
+    rows for a first sublayer that reads the residual stream as it is."""
     R, W = out.shape
     if not out.is_cuda:
-        out.copy_(embed[ids[:R].long()].float())
+        out.copy_(embed[ids[:R].long()].float() * scale)
         if h_out is not None:
             h_out[:R] = out.to(h_out.dtype)
         return out
@@ -229,7 +238,8 @@ def embed_rows(embed, ids, out, h_out=None):
         assert h_out.dtype == embed.dtype and h_out.shape[1] == W and h_out.shape[0] >= R
         ldh = h_out.stride(0)
     _chk(lib().p2p_sm_embed_rows(embed.data_ptr(), ids.data_ptr(), out.data_ptr(),
-                                 _lib.ptr(h_out), ldh, R, W, _f32(embed), _st(out)), "embed_rows")
+                                 _lib.ptr(h_out), ldh, R, W, scale, _f32(embed), _st(out)),
+         "embed_rows")
     return out
 
 
@@ -327,6 +337,65 @@ def add_norm(x, a, b=None, eps: float = 0.0, next_w=None, next_out=None):
     return x
 
 
+def add_norm2(x, a=None, b=None, rows=None, vec=None, eps: float = 0.0, w1=None, out1=None,
+              w2=None, out2=None):
+    """x += a + b + rows + vec on the fp32 residual x (every addend optional; a, b activation
+    typed [R, n], rows fp32 [R, n], vec fp32 [n]; they are summed in fp32 before they meet x),
+    then up to two normed copies of the updated rows in the same pass,
+    out_i = x / sqrt(mean(x^2) + eps) * w_i, each w_i fp32 with n numbers or a single one for
+    all channels: the inputs of two sublayers that read the same rows through norms of
+    their own."""
+    R, n = x.shape
+    if (w1 is None) != (out1 is None) or (w2 is None) != (out2 is None) or (w2 is not None and w1 is None):
+        raise ValueError("add_norm2: a norm weight goes with its output, the first before the second")
+    if not x.is_cuda:
+        y = None
+        for t in (a, b, rows):
+            if t is not None:
+                y = t[:R].float() if y is None else y + t[:R].float()
+        if vec is not None:
+            y = vec if y is None else y + vec
+        if y is not None:
+            x += y
+        for w, o in ((w1, out1), (w2, out2)):
+            if w is not None:
+                o[:R] = (_rms(x, eps) * w).to(o.dtype)
+        return x
+    assert x.dtype == torch.float32 and x.is_contiguous()
+    lda = ldb = 0
+    if a is not None:
+        _rows2d(a, "a")
+        assert a.shape[1] == n and a.shape[0] >= R
+        lda = a.stride(0)
+    if b is not None:
+        _rows2d(b, "b")
+        assert a is not None and b.shape[1] == n and b.shape[0] >= R and b.dtype == a.dtype
+        ldb = b.stride(0)
+    if rows is not None:
+        assert rows.dtype == torch.float32 and rows.is_contiguous() and rows.shape == x.shape
+    if vec is not None:
+        _vec(vec, n, "vec")
+    ld1 = ld2 = 0
+    for w, o, nm in ((w1, out1, "w1"), (w2, out2, "w2")):
+        if w is not None:
+            assert w.dtype == torch.float32 and w.is_contiguous() and w.numel() in (1, n), nm
+            _rows2d(o, "out")
+            assert o.shape[1] == n and o.shape[0] >= R and o.dtype == out1.dtype
+            assert a is None or o.dtype == a.dtype
+    if out1 is not None:
+        ld1 = out1.stride(0)
+    if out2 is not None:
+        ld2 = out2.stride(0)
+    act = a if a is not None else out1
+    _chk(lib().p2p_sm_add_norm2(x.data_ptr(), _lib.ptr(a), lda, _lib.ptr(b), ldb, _lib.ptr(rows),
+                                _lib.ptr(vec), R, n, eps, _lib.ptr(w1),
+                                1 if w1 is not None and w1.numel() > 1 else 0, _lib.ptr(out1), ld1,
+                                _lib.ptr(w2), 1 if w2 is not None and w2.numel() > 1 else 0,
+                                _lib.ptr(out2), ld2, _f32(act) if act is not None else 1, _st(x)),
+         "add_norm2")
+    return x
+
+
 # ------------------------------------------------------------------ pointwise
 def tanh_(x):
     if not x.is_cuda:
@@ -338,19 +407,23 @@ def tanh_(x):
     return x
 
 
-def sigmoid_gate(o, g, out, H: int, V: int):
-    """out[r, h*V + v] = o[h, r, v] * sigmoid(g[r, h*V + v]); o is any [H, R, V] view whose
-    last stride is 1."""
+def sigmoid_gate(o, g, out, H: int, V: int, per_head: bool = False):
+    """out[r, h*V + v] = o[h, r, v] * sigmoid(g[r, h*V + v]), or with ``per_head`` one gate for
+    all channels of a head, sigmoid(g[r, h]); o is any [H, R, V] view whose last stride is 1."""
     R = g.shape[0]
     if not g.is_cuda:
-        out.copy_((o.float().permute(1, 0, 2).reshape(R, H * V) * torch.sigmoid(g.float())).to(out.dtype))
+        gg = torch.sigmoid(g.float())
+        if per_head:
+            gg = gg[:, :H].repeat_interleave(V, 1)
+        out.copy_((o.float().permute(1, 0, 2).reshape(R, H * V) * gg).to(out.dtype))
         return out
     _rows2d(g, "g")
     _rows2d(out, "out")
     assert o.shape == (H, R, V) and o.stride(2) == 1 and o.dtype == g.dtype == out.dtype
+    assert g.shape[1] >= (H if per_head else H * V)
     _chk(lib().p2p_sm_sigmoid_gate(o.data_ptr(), o.stride(0), o.stride(1), g.data_ptr(),
-                                   g.stride(0), out.data_ptr(), out.stride(0), R, H, V, _f32(g),
-                                   _st(g)), "sigmoid_gate")
+                                   g.stride(0), out.data_ptr(), out.stride(0), R, H, V,
+                                   1 if per_head else 0, _f32(g), _st(g)), "sigmoid_gate")
     return out
 
 
@@ -608,7 +681,10 @@ def latent_attn(qa, cache, block_tables, row_ent, pos, sink, scale: float, win: 
     (W_uk^T q per head); cache [tokens, rank] one layer's latent pool, token t of a sequence
     at block_tables[e, t // page] * page + t % page.  out [H, R, rank] = sum_j p_j c_j with
     p = softmax over {sink_h} U {scale * qa . c_j : 0 <= pos - j < win}, the sink term having
-    no value.  units: ``make_units(entries, latent_rows_per_wave(H))`` on the device; with
+    no value (sink None: an ordinary softmax over the visible keys).  A layer whose keys have a
+    part outside the latent (a rotated part shared by the heads) appends it to the cached row and
+    the matching query part to qa; the columns of out beyond the latent are then not used.
+    units: ``make_units(entries, latent_rows_per_wave(H))`` on the device; with
     it, bf16 inputs run on the matrix cores (``latent_mfma_ok``).  max_keys: an upper bound of
     the keys any row sees (host side; lets a step of few rows split its windows)."""
     H, R, rank = qa.shape
@@ -621,9 +697,9 @@ def latent_attn(qa, cache, block_tables, row_ent, pos, sink, scale: float, win: 
             tok = bt[int(row_ent[r])][j // page] * page + j % page
             c = cache[tok].float()                                  # [n, rank]
             s = (qa[:, r].float() @ c.T) * scale                    # [H, n]
-            m = torch.maximum(s.max(-1).values, sink)
+            m = s.max(-1).values if sink is None else torch.maximum(s.max(-1).values, sink)
             e = torch.exp(s - m[:, None])
-            den = e.sum(-1) + torch.exp(sink - m)
+            den = e.sum(-1) if sink is None else e.sum(-1) + torch.exp(sink - m)
             out[:, r] = ((e / den[:, None]) @ c).to(out.dtype)
         return out
     assert qa.stride(2) == 1 and out.stride(2) == 1 and out.shape == qa.shape
@@ -631,7 +707,8 @@ def latent_attn(qa, cache, block_tables, row_ent, pos, sink, scale: float, win: 
     assert cache.dim() == 2 and cache.is_contiguous() and cache.shape[1] == rank
     assert block_tables.dtype == torch.int32 and block_tables.is_contiguous()
     assert row_ent.dtype == torch.int32 and pos.dtype == torch.int32
-    _vec(sink, H, "sink")
+    if sink is not None:
+        _vec(sink, H, "sink")
     if units is not None and latent_mfma_ok(qa, cache):
         assert units.dtype == torch.int32 and units.is_contiguous() and units.shape[1] == 2
         # few row groups with long windows (decode): cut every window into runs of key tiles
@@ -651,7 +728,7 @@ def latent_attn(qa, cache, block_tables, row_ent, pos, sink, scale: float, win: 
                                            cache.data_ptr(), block_tables.data_ptr(),
                                            block_tables.shape[1], row_ent.data_ptr(),
                                            pos.data_ptr(), units.data_ptr(), units.shape[0],
-                                           sink.data_ptr(), scale, win, out.data_ptr(),
+                                           _lib.ptr(sink), scale, win, out.data_ptr(),
                                            out.stride(0), out.stride(1), H, rank, page, splits,
                                            _lib.ptr(part), _st(qa)),
              "latent_attn_mfma")
@@ -660,7 +737,7 @@ def latent_attn(qa, cache, block_tables, row_ent, pos, sink, scale: float, win: 
         raise ValueError("latent_attn: %d heads x latent %d exceed the kernel's tile" % (H, rank))
     _chk(lib().p2p_sm_latent_attn(qa.data_ptr(), qa.stride(0), qa.stride(1), cache.data_ptr(),
                                   block_tables.data_ptr(), block_tables.shape[1],
-                                  row_ent.data_ptr(), pos.data_ptr(), sink.data_ptr(), scale,
+                                  row_ent.data_ptr(), pos.data_ptr(), _lib.ptr(sink), scale,
                                   win, out.data_ptr(), out.stride(0), out.stride(1), R, H, rank,
                                   page, _f32(qa), _st(qa)), "latent_attn")
     return out
@@ -744,15 +821,17 @@ def relu2_gate(u, g, out):
     return out
 
 
-def softcap(y, cap: float, out):
-    """out = cap * tanh(y / cap) as fp32 (y: activation-typed or fp32 logits)."""
+def softcap(y, cap: float, out, scale: float = 1.0):
+    """out = cap * tanh(scale * y / cap) as fp32 (y: activation-typed or fp32 logits); cap 0:
+    out = scale * y."""
     if not y.is_cuda:
-        out.copy_(cap * torch.tanh(y.float() / cap))
+        z = y.float() * scale
+        out.copy_(cap * torch.tanh(z / cap) if cap else z)
         return out
     _rows2d(y, "y")
     assert out.dtype == torch.float32 and out.is_contiguous() and out.shape == y.shape
     _chk(lib().p2p_sm_softcap(y.data_ptr(), y.stride(0), out.data_ptr(), y.shape[0], y.shape[1],
-                              cap, _f32(y), _st(y)), "softcap")
+                              cap, scale, _f32(y), _st(y)), "softcap")
     return out
 
 
@@ -773,6 +852,65 @@ def rope_inv_freq(base: float, dims: int, device, scaling: dict | None = None) -
         mid = (1.0 - s) * f / fac + s * f
         f = torch.where(wl < orig / hi, f, torch.where(wl > orig / lo, f / fac, mid))
     return f.float().to(device)
+
+
+def rope_rows(src, heads: int, src_hs: int, inv_freq, pos, dst, dst_hs: int, out_rows=None):
+    """Rotary positions on a stretch of channels: for every row r and head h < heads the
+    pairs (2i, 2i+1), i < len(inv_freq), of src[r, h*src_hs : ...] are turned by the angle
+    pos[r] * inv_freq[i], (a, b) -> (a cos - b sin, b cos + a sin) in fp32, and written to
+    dst[o(r), h*dst_hs : ...]; o(r) = out_rows[r] (a scatter, e.g. into a paged pool) or r.
+    src and dst are 2-d views that start at the first rotated channel of head 0 (last stride
+    1; a head may lie anywhere from there, also beyond the view's own width)."""
+    R = src.shape[0]
+    nrot = inv_freq.numel()
+    if nrot == 0 or heads == 0:
+        return dst
+    if not src.is_cuda:
+        ang = pos[:R].float()[:, None] * inv_freq[None, :]
+        c, sn = torch.cos(ang), torch.sin(ang)
+        ro = torch.arange(R) if out_rows is None else out_rows[:R].long()
+        sv = torch.as_strided(src, (R, heads, 2 * nrot), (src.stride(0), src_hs, 1), src.storage_offset())
+        dv = torch.as_strided(dst, (dst.shape[0], heads, 2 * nrot), (dst.stride(0), dst_hs, 1),
+                              dst.storage_offset())
+        a, b = sv[:, :, 0::2].float(), sv[:, :, 1::2].float()
+        res = torch.stack([a * c[:, None] - b * sn[:, None], b * c[:, None] + a * sn[:, None]], -1)
+        dv[ro] = res.reshape(R, heads, 2 * nrot).to(dst.dtype)
+        return dst
+    assert src.dim() == 2 and dst.dim() == 2 and src.stride(1) == 1 and dst.stride(1) == 1
+    assert src.dtype == dst.dtype and pos.dtype == torch.int32
+    assert inv_freq.dtype == torch.float32 and inv_freq.is_contiguous()
+    assert out_rows is None or (out_rows.dtype == torch.int32 and out_rows.numel() >= R)
+    assert pos.numel() >= R
+    _chk(lib().p2p_sm_rope_rows(src.data_ptr(), src.stride(0), heads, src_hs, inv_freq.data_ptr(),
+                                nrot, pos.data_ptr(), _lib.ptr(out_rows), dst.data_ptr(),
+                                dst.stride(0), dst_hs, R, _f32(src), _st(src)), "rope_rows")
+    return dst
+
+
+def qtemp_kv_store(proj, nq: int, nkv: int, coef: float, every: int, pos, cache_rows, pool, q_out):
+    """Prepares unrotated attention inputs from one projection buffer proj = [q (nq) | k and v
+    (nkv)]: q goes to q_out multiplied by the query temperature of its position p,
+    1 + coef * ln(floor((p + 1) / every) + 1) (fp32; coef 0: a plain copy), k | v go to the rows
+    ``cache_rows`` of the paged pool ([tokens, nkv])."""
+    R = q_out.shape[0]
+    if every < 1:
+        raise ValueError("query temperature step of %d positions" % every)
+    if not proj.is_cuda:
+        p = pos[:R].long()
+        temp = 1.0 + coef * torch.log((torch.div(p + 1, every, rounding_mode="floor") + 1).float())
+        q_out[:R] = (proj[:R, :nq].float() * temp[:, None]).to(q_out.dtype)
+        pool[cache_rows[:R].long()] = proj[:R, nq:nq + nkv].to(pool.dtype)
+        return q_out
+    _rows2d(proj, "proj")
+    _rows2d(q_out, "q_out")
+    assert proj.shape[1] >= nq + nkv and q_out.shape[1] == nq and q_out.dtype == proj.dtype
+    assert pool.dim() == 2 and pool.is_contiguous() and pool.shape[1] == nkv and pool.dtype == proj.dtype
+    assert pos.dtype == torch.int32 and cache_rows.dtype == torch.int32
+    _chk(lib().p2p_sm_qtemp_kv_store(proj.data_ptr(), proj.stride(0), nq, nkv, coef, every,
+                                     pos.data_ptr(), cache_rows.data_ptr(), pool.data_ptr(),
+                                     q_out.data_ptr(), q_out.stride(0), R, _f32(proj), _st(proj)),
+         "qtemp_kv_store")
+    return q_out
 
 
 def qk_norm_rope_store(proj, H: int, G: int, D: int, V: int, qw, kw, inv_freq, pos, cache_rows,
@@ -850,7 +988,8 @@ def window_mfma_ok(q, pool, D: int, V: int) -> bool:
 
 
 def window_attn(q, pool, block_tables, row_ent, pos, sink, scale: float, win: int, out, page: int,
-                H: int, G: int, D: int, V: int, units=None, max_keys=None, out_scale: float = 1.0):
+                H: int, G: int, D: int, V: int, units=None, max_keys=None, out_scale: float = 1.0,
+                softcap: float = 0.0, dist=None, gate=None):
     """Grouped-query attention over a paged key/value pool with a causal sliding window and a
     softmax sink.
 
@@ -860,6 +999,10 @@ def window_attn(q, pool, block_tables, row_ent, pos, sink, scale: float, win: in
     p = softmax over {sink_h} U {scale * q . k_j : 0 <= pos - j < win}; the sink has no value
     (sink None: an ordinary softmax over the visible keys);
     the result is multiplied by out_scale before it is rounded.
+    softcap c > 0: a score s becomes c * tanh(s / c).  dist = (r1, r2), fp32 [H] each: a key
+    d = pos - j positions back loses r1_h * ln(1 + r2_h * d) of its score (after the cap).
+    gate: a 2-d view [R, >= H] of the activation type; head h of row r leaves multiplied by
+    sigmoid(gate[r, h]).  Scores, cap, penalty, softmax and gate are fp32.
     units: ``make_units(entries, window_rows_per_wave(H // G))`` on the device; with it bf16
     inputs run on the matrix cores (``window_mfma_ok``)."""
     R = q.shape[0]
@@ -875,10 +1018,17 @@ def window_attn(q, pool, block_tables, row_ent, pos, sink, scale: float, win: in
             k = kv[:, :G * D].view(-1, G, D).repeat_interleave(HG, 1)       # [n, H, D]
             v = kv[:, G * D:].view(-1, G, V).repeat_interleave(HG, 1)
             s = torch.einsum("hd,nhd->hn", q[r].float().view(H, D), k) * scale
+            if softcap:
+                s = softcap * torch.tanh(s / softcap)
+            if dist is not None:
+                s = s - dist[0][:, None] * torch.log1p(dist[1][:, None] * (p - j).float()[None, :])
             m = s.max(-1).values if sink is None else torch.maximum(s.max(-1).values, sink)
             e = torch.exp(s - m[:, None])
             den = e.sum(-1) if sink is None else e.sum(-1) + torch.exp(sink - m)
-            out[r] = (torch.einsum("hn,nhv->hv", e / den[:, None], v).reshape(H * V) * out_scale).to(out.dtype)
+            o = torch.einsum("hn,nhv->hv", e / den[:, None], v)
+            if gate is not None:
+                o = o * torch.sigmoid(gate[r, :H].float())[:, None]
+            out[r] = (o.reshape(H * V) * out_scale).to(out.dtype)
         return out
     _rows2d(q, "q")
     _rows2d(out, "out")
@@ -891,6 +1041,16 @@ def window_attn(q, pool, block_tables, row_ent, pos, sink, scale: float, win: in
         _vec(sink, H, "sink")
     if win < 1:
         raise ValueError("window of %d keys" % win)
+    r1 = r2 = None
+    if dist is not None:
+        r1, r2 = dist
+        _vec(r1, H, "r1")
+        _vec(r2, H, "r2")
+    ldg = 0
+    if gate is not None:
+        _rows2d(gate, "gate")
+        assert gate.shape[0] >= R and gate.shape[1] >= H and gate.dtype == q.dtype
+        ldg = gate.stride(0)
     if units is not None and window_mfma_ok(q, pool, D, V):
         assert units.dtype == torch.int32 and units.is_contiguous() and units.shape[1] == 2
         U = units.shape[0]
@@ -910,12 +1070,14 @@ def window_attn(q, pool, block_tables, row_ent, pos, sink, scale: float, win: in
                                            row_ent.data_ptr(), pos.data_ptr(), units.data_ptr(), U,
                                            _lib.ptr(sink), scale, win, out.data_ptr(),
                                            out.stride(0), H, G, D, V, page, splits, _lib.ptr(part),
-                                           out_scale, _st(q)), "window_attn_mfma")
+                                           out_scale, softcap, _lib.ptr(r1), _lib.ptr(r2),
+                                           _lib.ptr(gate), ldg, _st(q)), "window_attn_mfma")
         return out
     _chk(lib().p2p_sm_window_attn(q.data_ptr(), q.stride(0), pool.data_ptr(),
                                   block_tables.data_ptr(), block_tables.shape[1],
                                   row_ent.data_ptr(), pos.data_ptr(), _lib.ptr(sink), scale, win,
                                   out.data_ptr(), out.stride(0), R, H, G, D, V, page, out_scale,
+                                  softcap, _lib.ptr(r1), _lib.ptr(r2), _lib.ptr(gate), ldg,
                                   _f32(q), _st(q)), "window_attn")
     return out
 
@@ -1108,10 +1270,15 @@ def mlstm_scan(proj, bi, bf, cap: float, normw, state, mstate, ent, ent_host, ou
 
 
 # ------------------------------------------------------------------ mixture of experts
+ROUTE_SCORES = {"sigmoid": 0, "softmax": 1, "top_softmax": 2}
+
+
 def group_route(h, wr, top: int, groups: int, keep: int, ids, wts, cnt, rows,
-                score: str = "sigmoid", corr=None, group_score: str = "top2"):
-    """Router with group-limited choice.  z = h wr^T in fp32 (wr fp32 [E, W]); the scores are
-    s = sigmoid(z) or (``score`` "softmax") softmax(z) over all E; the choice is made on
+                score: str = "sigmoid", corr=None, group_score: str = "top2", bias=None):
+    """Router with group-limited choice.  z = h wr^T (+ bias, fp32 [E]) in fp32 (wr fp32
+    [E, W]); the scores are s = sigmoid(z) or (``score`` "softmax") softmax(z) over all E, or
+    (``score`` "top_softmax") s = z for the choice and the weights are the softmax over the
+    chosen z only; the choice is made on
     c = s + corr (corr fp32 [E], optional).  The E experts are cut into ``groups`` contiguous
     blocks of equal size, a block is ranked by the sum of its two best c (``group_score``
     "top2") or by its best c ("max"), experts outside the ``keep`` best blocks are struck out;
@@ -1121,11 +1288,13 @@ def group_route(h, wr, top: int, groups: int, keep: int, ids, wts, cnt, rows,
     R = h.shape[0]
     E = wr.shape[0]
     per = E // groups
-    if score not in ("sigmoid", "softmax") or group_score not in ("top2", "max"):
+    if score not in ROUTE_SCORES or group_score not in ("top2", "max"):
         raise ValueError("group_route: score %r / group score %r" % (score, group_score))
     if not h.is_cuda:
         z = h[:R].float() @ wr.t()                                                # [R, E]
-        s = torch.sigmoid(z) if score == "sigmoid" else torch.softmax(z, -1)
+        if bias is not None:
+            z = z + bias
+        s = torch.sigmoid(z) if score == "sigmoid" else torch.softmax(z, -1) if score == "softmax" else z
         c = s if corr is None else s + corr
         gs = c.view(R, groups, per).topk(min(2, per) if group_score == "top2" else 1, dim=-1).values.sum(-1)
         best = gs.topk(keep, dim=-1).indices
@@ -1133,7 +1302,7 @@ def group_route(h, wr, top: int, groups: int, keep: int, ids, wts, cnt, rows,
         masked = torch.where(ok.repeat_interleave(per, 1), c, torch.full_like(c, -float("inf")))
         i = masked.topk(top, dim=-1).indices
         ids[:R] = i.to(torch.int32)
-        wts[:R] = s.gather(1, i)
+        wts[:R] = s.gather(1, i) if score != "top_softmax" else torch.softmax(s.gather(1, i), -1)
         cnt.zero_()
         for slot, e in enumerate(i.reshape(-1).tolist()):
             rows[e, int(cnt[e])] = slot
@@ -1146,6 +1315,8 @@ def group_route(h, wr, top: int, groups: int, keep: int, ids, wts, cnt, rows,
         raise ValueError("group_route: %d experts > 1024" % E)
     if corr is not None:
         _vec(corr, E, "corr")
+    if bias is not None:
+        _vec(bias, E, "bias")
     assert ids.dtype == torch.int32 and ids.is_contiguous() and ids.shape == (R, top)
     assert wts.dtype == torch.float32 and wts.is_contiguous() and wts.shape == (R, top)
     assert cnt.dtype == torch.int32 and cnt.numel() == E
@@ -1153,10 +1324,10 @@ def group_route(h, wr, top: int, groups: int, keep: int, ids, wts, cnt, rows,
         and rows.shape[1] >= R * top
     cnt.zero_()
     _chk(lib().p2p_sm_group_route(h.data_ptr(), h.stride(0), wr.data_ptr(), R, h.shape[1], E, top,
-                                  groups, keep, 1 if score == "softmax" else 0, _lib.ptr(corr),
+                                  groups, keep, ROUTE_SCORES[score], _lib.ptr(corr),
                                   1 if group_score == "max" else 0, ids.data_ptr(),
                                   wts.data_ptr(), cnt.data_ptr(), rows.data_ptr(), rows.stride(0),
-                                  _f32(h), _st(h)), "group_route")
+                                  _lib.ptr(bias), _f32(h), _st(h)), "group_route")
     return ids, wts
 
 
@@ -1172,7 +1343,7 @@ def interleave_gate_up(gate, up):
 
 
 def expert_gemm(x, x_div: int, w, cnt, rows, out, total_slots: int, act_limit=None,
-                act_alpha: float = 1.702, relu2: bool = False):
+                act_alpha: float = 1.702, relu2: bool = False, silu_glu: bool = False):
     """Per expert e and each of its routed slots s = rows[e, i] (i < cnt[e]):
     out[s] = x[s // x_div] @ w[e]^T.  w [E, N, K] (activation type), x [*, K], out [slots, N].
     total_slots: the slots over all experts (every slot is in exactly one list; the grid is
@@ -1181,12 +1352,13 @@ def expert_gemm(x, x_div: int, w, cnt, rows, out, total_slots: int, act_limit=No
     act_limit: w = ``interleave_gate_up(gate, up)`` and out [slots, N/2] receives
     min(g, L) * sigmoid(alpha * min(g, L)) * (clamp(u, -L, L) + 1) of the two products (fp32
     before the rounding) instead of the products themselves.
+    silu_glu: w = ``interleave_gate_up(gate, up)`` and out [slots, N/2] receives g * sigmoid(g) * u.
     relu2: out receives relu(.)^2 of every product (an ungated unit; fp32 before the rounding).
     cnt may list more experts than w holds (experts without weights): their slots are left
     out."""
     E, N, K = w.shape
-    fused = act_limit is not None
-    if fused and relu2:
+    fused = act_limit is not None or silu_glu
+    if (act_limit is not None) + bool(relu2) + bool(silu_glu) > 1:
         raise ValueError("expert_gemm: one activation at a time")
     if not x.is_cuda:
         for e in range(E):
@@ -1194,7 +1366,10 @@ def expert_gemm(x, x_div: int, w, cnt, rows, out, total_slots: int, act_limit=No
             if not sl.numel():
                 continue
             y = torch.nn.functional.linear(x[sl // x_div].float(), w[e].float())
-            if fused:
+            if silu_glu:
+                y = y.view(-1, N // 32, 2, 16)
+                y = (y[:, :, 0] * torch.sigmoid(y[:, :, 0]) * y[:, :, 1]).reshape(-1, N // 2)
+            elif fused:
                 y = y.view(-1, N // 32, 2, 16)
                 g = torch.clamp(y[:, :, 0], max=act_limit)
                 u = torch.clamp(y[:, :, 1], -act_limit, act_limit)
@@ -1211,8 +1386,10 @@ def expert_gemm(x, x_div: int, w, cnt, rows, out, total_slots: int, act_limit=No
         raise ValueError("fused expert activation needs gate / up widths that are multiples of 16")
     _chk(lib().p2p_sm_expert_gemm(x.data_ptr(), x.stride(0), x_div, w.data_ptr(), cnt.data_ptr(),
                                   rows.data_ptr(), rows.stride(0), out.data_ptr(), out.stride(0),
-                                  E, N, K, total_slots, 1 if fused else 2 if relu2 else 0,
-                                  float(act_limit) if fused else 0.0, act_alpha, _f32(x), _st(x)),
+                                  E, N, K, total_slots,
+                                  3 if silu_glu else 1 if fused else 2 if relu2 else 0,
+                                  float(act_limit) if act_limit is not None else 0.0, act_alpha,
+                                  _f32(x), _st(x)),
          "expert_gemm")
     return out
 

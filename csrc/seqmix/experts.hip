@@ -39,20 +39,22 @@ __device__ __forceinline__ void wave_sync() {
   __builtin_amdgcn_wave_barrier();
 }
 
-// score: 0 sigmoid, 1 softmax over all experts.  corr (optional, [E]): added to the scores for
-// the choice only.  gscore: a group is ranked by 0 the sum of its two best choice scores, 1 its
+// score: 0 sigmoid, 1 softmax over all experts, 2 the logits themselves for the choice and the
+// softmax over the chosen logits as weights.  bias (optional, [E]): added to the logits.
+// corr (optional, [E]): added to the scores for the choice only.  gscore: a group is ranked by 0 the sum of its two best choice scores, 1 its
 // best choice score.
 template <typename T>
 __global__ void __launch_bounds__(256)
 group_route_k(const T* __restrict__ h, int ldh, const float* __restrict__ wr, int W, int E, int top,
               int groups, int keep, int score, const float* __restrict__ corr, int gscore,
               int* __restrict__ ids, float* __restrict__ wts, int* __restrict__ cnt,
-              int* __restrict__ rows, int ldr) {
+              int* __restrict__ rows, int ldr, const float* __restrict__ bias) {
   extern __shared__ float smem[];
   float* sh = smem;          // [W] the row in fp32
   float* ss = sh + W;        // [E] scores (the weights of the chosen)
   float* sc = ss + E;        // [E] choice scores; -inf marks "cannot be chosen (any more)"
   float* sgs = sc + E;       // [groups] group scores
+  float* stop = sgs + groups;   // [top] the chosen logits (score 2)
   const int r = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
   for (int i = threadIdx.x; i < W; i += blockDim.x) sh[i] = ldf(h, (size_t)r * ldh + i);
   __syncthreads();
@@ -76,6 +78,12 @@ group_route_k(const T* __restrict__ h, int ldh, const float* __restrict__ wr, in
     d2 = wave_sum(d2);
     d3 = wave_sum(d3);
     if (lane == 0) {
+      if (bias) {
+        d0 += bias[e0];
+        d1 += bias[min(e0 + 1, E - 1)];
+        d2 += bias[min(e0 + 2, E - 1)];
+        d3 += bias[min(e0 + 3, E - 1)];
+      }
       ss[e0] = score ? d0 : sigmoidf_(d0);
       if (e0 + 1 < E) ss[e0 + 1] = score ? d1 : sigmoidf_(d1);
       if (e0 + 2 < E) ss[e0 + 2] = score ? d2 : sigmoidf_(d2);
@@ -84,7 +92,7 @@ group_route_k(const T* __restrict__ h, int ldh, const float* __restrict__ wr, in
   }
   __syncthreads();
   if (wave != 0) return;
-  if (score) {   // softmax over all experts
+  if (score == 1) {   // softmax over all experts
     float mx = -INFINITY;
     for (int e = lane; e < E; e += 64) mx = fmaxf(mx, ss[e]);
 #pragma unroll
@@ -140,11 +148,22 @@ group_route_k(const T* __restrict__ h, int ldh, const float* __restrict__ wr, in
       sc[bi] = -INFINITY;
       int slot = r * top + k;
       ids[slot] = bi;
-      wts[slot] = ss[bi];
+      if (score == 2) stop[k] = ss[bi];
+      else wts[slot] = ss[bi];
       int at = atomicAdd(&cnt[bi], 1);
       rows[(size_t)bi * ldr + at] = slot;
     }
     wave_sync();
+  }
+  if (score == 2) {   // the weights become the softmax over the chosen logits
+    float mx = -INFINITY;
+    for (int k = lane; k < top; k += 64) mx = fmaxf(mx, stop[k]);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+    float sum = 0.0f;
+    for (int k = lane; k < top; k += 64) sum += expf(stop[k] - mx);
+    sum = wave_sum(sum);
+    for (int k = lane; k < top; k += 64) wts[r * top + k] = expf(stop[k] - mx) / sum;
   }
 }
 
@@ -209,6 +228,11 @@ __device__ __forceinline__ float expert_act(float g, float u, float limit, float
   g = fminf(g, limit);
   u = fminf(fmaxf(u, -limit), limit);
   return g * sigmoidf_(alpha * g) * (u + 1.0f);
+}
+
+// epi = 3: the same layout with y = g * sigmoid(g) * u
+__device__ __forceinline__ float glu_epi(float g, float u, int epi, float limit, float alpha) {
+  return epi == 3 ? g * sigmoidf_(g) * u : expert_act(g, u, limit, alpha);
 }
 
 // epi = 2: an ungated unit, every product passes relu(.)^2; epi = 0: the products themselves
@@ -288,13 +312,13 @@ expert_gemm_mfma_k(const bf16* __restrict__ x, int ldx, int x_div, const bf16* _
   for (int i = 0; i < 4; i++) {
     int so = __shfl(slot, quad * 4 + i, 64);
     if (so < 0) continue;
-    if (epi == 1) {
+    if (epi == 1 || epi == 3) {
 #pragma unroll
       for (int t = 0; t < 4; t += 2) {
         int n = n0 + t * 16;
         if (n + 16 + n16 < N)
           out[(size_t)so * ldo + n / 2 + n16] =
-              __float2bfloat16(expert_act(acc[t][i], acc[t + 1][i], limit, alpha));
+              __float2bfloat16(glu_epi(acc[t][i], acc[t + 1][i], epi, limit, alpha));
       }
       continue;
     }
@@ -396,13 +420,13 @@ expert_gemm_mfma_big_k(const bf16* __restrict__ x, int ldx, int x_div, const bf1
     for (int i = 0; i < 4; i++) {
       int so = sslot[wm + a * 16 + quad * 4 + i];
       if (so < 0) continue;
-      if (epi == 1) {
+      if (epi == 1 || epi == 3) {
 #pragma unroll
         for (int b = 0; b < 4; b += 2) {
           int n = n0 + wn + b * 16;
           if (n + 16 + n16 < N)
             out[(size_t)so * ldo + n / 2 + n16] =
-                __float2bfloat16(expert_act(acc[a][b][i], acc[a][b + 1][i], limit, alpha));
+                __float2bfloat16(glu_epi(acc[a][b][i], acc[a][b + 1][i], epi, limit, alpha));
         }
         continue;
       }
@@ -465,12 +489,13 @@ expert_gemm_fma_k(const T* __restrict__ x, int ldx, int x_div, const T* __restri
   for (int a = 0; a < 2; a++) {
     int s = sslot[ty * 2 + a];
     if (s < 0) continue;
-    if (epi == 1) {
+    if (epi == 1 || epi == 3) {
 #pragma unroll
       for (int u = 0; u < 4; u += 2) {
         int n = n0 + 16 * u;
         if (n + 16 + tx < N)
-          stf(out, (size_t)s * ldo + n / 2 + tx, expert_act(acc[a][u], acc[a][u + 1], limit, alpha));
+          stf(out, (size_t)s * ldo + n / 2 + tx,
+              glu_epi(acc[a][u], acc[a][u + 1], epi, limit, alpha));
       }
       continue;
     }
@@ -505,16 +530,17 @@ extern "C" {
 // cnt must be zero on entry
 int p2p_sm_group_route(const void* h, int ldh, const float* wr, int R, int W, int E, int top,
                        int groups, int keep, int score, const float* corr, int gscore, int* ids,
-                       float* wts, int* cnt, int* rows, int ldr, int f32, hipStream_t st) {
+                       float* wts, int* cnt, int* rows, int ldr, const float* bias, int f32,
+                       hipStream_t st) {
   if (R <= 0) return 0;
   if (E < 1 || groups < 1 || E % groups || keep < 1 || keep > groups || top < 1 ||
       top > keep * (E / groups) || ldr < R * top)
     return (int)hipErrorInvalidValue;
-  size_t shm = (size_t)(W + 2 * E + groups) * 4;
+  size_t shm = (size_t)(W + 2 * E + groups + top) * 4;
   if (shm > 64 * 1024) return (int)hipErrorInvalidValue;
   SM_DISPATCH_T(f32, hipLaunchKernelGGL(group_route_k<T>, dim3(R), dim3(256), shm, st,
                                          (const T*)h, ldh, wr, W, E, top, groups, keep, score, corr,
-                                         gscore, ids, wts, cnt, rows, ldr));
+                                         gscore, ids, wts, cnt, rows, ldr, bias));
   return (int)hipGetLastError();
 }
 
@@ -526,7 +552,8 @@ int p2p_sm_expert_gemm(const void* x, int ldx, int x_div, const void* w, const i
                        int total_slots, int epi, float limit, float alpha, int f32,
                        hipStream_t st) {
   if (total_slots <= 0 || E <= 0) return 0;
-  if (x_div < 1 || N < 1 || K < 1 || (epi == 1 && N % 32)) return (int)hipErrorInvalidValue;
+  if (x_div < 1 || N < 1 || K < 1 || ((epi == 1 || epi == 3) && N % 32))
+    return (int)hipErrorInvalidValue;
   if (!f32 && K % 8 == 0 && ldx % 8 == 0 && ((size_t)x & 15) == 0 && ((size_t)w & 15) == 0) {
     if (total_slots >= 64 * E) {   // prompts: the large tile
       int tmp = (((total_slots + 127) / 128 + E) + 7) & ~7;

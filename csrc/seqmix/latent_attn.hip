@@ -27,7 +27,7 @@ latent_attn_k(const T* __restrict__ qa, long sqh, long sqr, const T* __restrict_
   int H = min(HG, Hall - h0);            // heads of this block
   qa += (size_t)h0 * sqh;
   out += (size_t)h0 * soh;
-  sink += h0;
+  if (sink) sink += h0;
   float* sq = smem;                      // [H][rank]
   float* sc = sq + HG * rank;            // [TK][rank + 1]
   float* sp = sc + TK * ldc;             // [H][TK]
@@ -43,8 +43,8 @@ latent_attn_k(const T* __restrict__ qa, long sqh, long sqr, const T* __restrict_
     sq[idx] = ldf(qa, (size_t)h * sqh + (size_t)r * sqr + c);
   }
   if (tid < H) {
-    sm_[tid] = sink[tid];
-    sl[tid] = 1.0f;
+    sm_[tid] = sink ? sink[tid] : -1e30f;   // no sink: an ordinary softmax
+    sl[tid] = sink ? 1.0f : 0.0f;
   }
   float acc[LA_ACC];
 #pragma unroll

@@ -1,7 +1,8 @@
 // Latent attention on the matrix cores (bf16 activations, fp32 scores / softmax / sums).
 // Same inputs and outputs as latent_attn.hip: queries arrive in latent space (qa = W_uk^T q), a score
 // is scale * qa . c_j over the cached latents of the causal sliding window, the softmax
-// denominator also holds exp(sink_h), and the result is sum_j p_j c_j per head.
+// denominator also holds exp(sink_h) (no sink given: an ordinary softmax), and the result is
+// sum_j p_j c_j per head.
 //
 // Every head attends to the same latents, so (row, head) pairs are the M dimension: one
 // wavefront owns 16 pairs -- RW consecutive rows of one sequence portion x HS head slots --
@@ -66,8 +67,9 @@ latent_attn_mfma_k(const bf16* __restrict__ qa, long sqh, long sqr, const bf16* 
   }
   __syncthreads();
 
-  float m_run = pvalid ? (first ? sink[ph] : -1e30f) : 0.0f;
-  float l_part = (pvalid && quad == 0 && first) ? 1.0f : 0.0f;
+  const bool sunk = first && sink != nullptr;   // no sink: an ordinary softmax
+  float m_run = pvalid ? (sunk ? sink[ph] : -1e30f) : 0.0f;
+  float l_part = (pvalid && quad == 0 && sunk) ? 1.0f : 0.0f;
   f32x4 acc[NT];
 #pragma unroll
   for (int t = 0; t < NT; t++) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};

@@ -193,14 +193,89 @@ __global__ void add_norm_k(float* __restrict__ x, const T* __restrict__ a, int l
     stf(h, (size_t)r * ldh + i, xr[i] * r2 * w2[i]);
 }
 
-// out[r] = embed[ids[r]] as fp32, and (optionally) the same row in the activation type
+// x += a + b + rows + vec on the fp32 residual (each addend optional; a, b activation typed,
+// rows fp32 [R, n], vec fp32 [n]; summed first, in fp32), then up to two normed copies of the
+// updated row, h_i = x / sqrt(mean(x^2) + eps) * w_i, where w_i is a vector (ws_i = 1) or one
+// number for all channels (ws_i = 0): two sublayers that read the same row through norms of
+// their own get their inputs from one pass over it.
+template <typename T>
+__global__ void add_norm2_k(float* __restrict__ x, const T* __restrict__ a, int lda,
+                            const T* __restrict__ b, int ldb, const float* __restrict__ rows,
+                            const float* __restrict__ vec, int n, float eps,
+                            const float* __restrict__ w1, int ws1, T* __restrict__ h1, int ld1,
+                            const float* __restrict__ w2, int ws2, T* __restrict__ h2, int ld2) {
+  __shared__ float red[16];
+  int r = blockIdx.x;
+  const T* ar = a ? a + (size_t)r * lda : nullptr;
+  const T* br = b ? b + (size_t)r * ldb : nullptr;
+  const float* er = rows ? rows + (size_t)r * n : nullptr;
+  float* xr = x + (size_t)r * n;
+  const bool adds = ar || br || er || vec;
+  if (n <= NV * (int)blockDim.x) {
+    // every load goes out before the first store
+    float xv[NV];
+    float s2 = 0.0f;
+#pragma unroll
+    for (int k = 0; k < NV; k++) {
+      int i = threadIdx.x + k * blockDim.x;
+      bool ok = i < n;
+      int ic = ok ? i : 0;
+      float y = 0.0f;
+      if (ar) y += ldf(ar, ic);
+      if (br) y += ldf(br, ic);
+      if (er) y += er[ic];
+      if (vec) y += vec[ic];
+      xv[k] = ok ? xr[ic] + y : 0.0f;
+    }
+#pragma unroll
+    for (int k = 0; k < NV; k++) {
+      int i = threadIdx.x + k * blockDim.x;
+      if (adds && i < n) xr[i] = xv[k];
+      s2 += xv[k] * xv[k];
+    }
+    if (!w1) return;
+    s2 = block_sum(s2, red);
+    float r2 = 1.0f / sqrtf(s2 / (float)n + eps);
+#pragma unroll
+    for (int k = 0; k < NV; k++) {
+      int i = threadIdx.x + k * blockDim.x;
+      if (i < n) {
+        stf(h1, (size_t)r * ld1 + i, xv[k] * r2 * w1[ws1 ? i : 0]);
+        if (w2) stf(h2, (size_t)r * ld2 + i, xv[k] * r2 * w2[ws2 ? i : 0]);
+      }
+    }
+    return;
+  }
+  float s2 = 0.0f;
+  for (int i = threadIdx.x; i < n; i += blockDim.x) {
+    float y = 0.0f;
+    if (ar) y += ldf(ar, i);
+    if (br) y += ldf(br, i);
+    if (er) y += er[i];
+    if (vec) y += vec[i];
+    float v = xr[i] + y;
+    if (adds) xr[i] = v;
+    s2 += v * v;
+  }
+  if (!w1) return;
+  s2 = block_sum(s2, red);
+  float r2 = 1.0f / sqrtf(s2 / (float)n + eps);
+  for (int i = threadIdx.x; i < n; i += blockDim.x) {   // each thread re-reads its own writes
+    float v = xr[i];
+    stf(h1, (size_t)r * ld1 + i, v * r2 * w1[ws1 ? i : 0]);
+    if (w2) stf(h2, (size_t)r * ld2 + i, v * r2 * w2[ws2 ? i : 0]);
+  }
+}
+
+// out[r] = embed[ids[r]] * scale as fp32, and (optionally) the same row in the activation type
 template <typename T>
 __global__ void embed_rows_k(const T* __restrict__ embed, const int* __restrict__ ids,
-                             float* __restrict__ out, T* __restrict__ h, int ldh, int W) {
+                             float* __restrict__ out, T* __restrict__ h, int ldh, int W,
+                             float scale) {
   int r = blockIdx.x;
   size_t eo = (size_t)ids[r] * W;
   for (int i = threadIdx.x; i < W; i += blockDim.x) {
-    float v = ldf(embed, eo + i);
+    float v = ldf(embed, eo + i) * scale;
     out[(size_t)r * W + i] = v;
     if (h) stf(h, (size_t)r * ldh + i, v);
   }
@@ -264,10 +339,10 @@ __global__ void gate_norm_add_k(float* __restrict__ x, const T* __restrict__ y, 
 extern "C" {
 
 int p2p_sm_embed_rows(const void* embed, const int* ids, float* out, void* h, int ldh, int R,
-                      int W, int f32, hipStream_t st) {
+                      int W, float scale, int f32, hipStream_t st) {
   if (R <= 0) return 0;
   SM_DISPATCH_T(f32, hipLaunchKernelGGL(embed_rows_k<T>, dim3(R), dim3(256), 0, st,
-                                         (const T*)embed, ids, out, (T*)h, ldh, W));
+                                         (const T*)embed, ids, out, (T*)h, ldh, W, scale));
   return (int)hipGetLastError();
 }
 
@@ -318,6 +393,17 @@ int p2p_sm_norm_scale_add(float* x, const void* y, int ldy, const float* w, cons
   if (R <= 0) return 0;
   SM_DISPATCH_T(f32, hipLaunchKernelGGL(norm_scale_add_k<T>, dim3(R), dim3(256), 0, st, x,
                                          (const T*)y, ldy, w, ls, n, eps, w2, (T*)h, ldh));
+  return (int)hipGetLastError();
+}
+
+int p2p_sm_add_norm2(float* x, const void* a, int lda, const void* b, int ldb, const float* rows,
+                     const float* vec, int R, int n, float eps, const float* w1, int ws1, void* h1,
+                     int ld1, const float* w2, int ws2, void* h2, int ld2, int f32, hipStream_t st) {
+  if (R <= 0) return 0;
+  if ((w1 && !h1) || (w2 && (!h2 || !w1)) || (b && !a)) return (int)hipErrorInvalidValue;
+  SM_DISPATCH_T(f32, hipLaunchKernelGGL(add_norm2_k<T>, dim3(R), dim3(256), 0, st, x, (const T*)a,
+                                         lda, (const T*)b, ldb, rows, vec, n, eps, w1, ws1,
+                                         (T*)h1, ld1, w2, ws2, (T*)h2, ld2));
   return (int)hipGetLastError();
 }
 

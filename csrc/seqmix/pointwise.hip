@@ -14,12 +14,13 @@ __global__ void tanh_k(T* x, int ld, int n, int R) {
 // out[r, h * V + v] = o[h * soh + r * sor + v] * sigmoid(g[r * ldg + h * V + v])
 template <typename T>
 __global__ void sigmoid_gate_k(const T* __restrict__ o, long soh, long sor, const T* __restrict__ g,
-                               int ldg, T* __restrict__ out, int ldo, int H, int V) {
+                               int ldg, T* __restrict__ out, int ldo, int H, int V,
+                               int per_head) {
   int c = blockIdx.x * blockDim.x + threadIdx.x, r = blockIdx.y;
   if (c >= H * V) return;
   int h = c / V, v = c % V;
   float x = ldf(o, (size_t)h * soh + (size_t)r * sor + v);
-  stf(out, (size_t)r * ldo + c, x * sigmoidf_(ldf(g, (size_t)r * ldg + c)));
+  stf(out, (size_t)r * ldo + c, x * sigmoidf_(ldf(g, (size_t)r * ldg + (per_head ? h : c))));
 }
 
 template <typename T>
@@ -63,9 +64,11 @@ __global__ void relu2_gate_k(const T* __restrict__ u, int ld, const T* __restric
 
 template <typename T>
 __global__ void softcap_k(const T* __restrict__ y, int ld, float* __restrict__ out, int n,
-                          float cap) {
+                          float cap, float scale) {
   int c = blockIdx.x * blockDim.x + threadIdx.x, r = blockIdx.y;
-  if (c < n) out[(size_t)r * n + c] = cap * tanhf(ldf(y, (size_t)r * ld + c) / cap);
+  if (c >= n) return;
+  float z = ldf(y, (size_t)r * ld + c) * scale;
+  out[(size_t)r * n + c] = cap > 0.0f ? cap * tanhf(z / cap) : z;
 }
 
 extern "C" {
@@ -88,11 +91,12 @@ int p2p_sm_relu2_gate(const void* u, int ld, const void* gt, int ldg, void* out,
   return (int)hipGetLastError();
 }
 
-int p2p_sm_softcap(const void* y, int ld, float* out, int R, int n, float cap, int f32,
-                   hipStream_t st) {
+int p2p_sm_softcap(const void* y, int ld, float* out, int R, int n, float cap, float scale,
+                   int f32, hipStream_t st) {
   if (R <= 0 || n <= 0) return 0;
   dim3 g((n + 255) / 256, R), b(256);
-  SM_DISPATCH_T(f32, hipLaunchKernelGGL(softcap_k<T>, g, b, 0, st, (const T*)y, ld, out, n, cap));
+  SM_DISPATCH_T(f32, hipLaunchKernelGGL(softcap_k<T>, g, b, 0, st, (const T*)y, ld, out, n, cap,
+                                         scale));
   return (int)hipGetLastError();
 }
 
@@ -104,11 +108,11 @@ int p2p_sm_tanh(void* x, int ld, int n, int R, int f32, hipStream_t st) {
 }
 
 int p2p_sm_sigmoid_gate(const void* o, long soh, long sor, const void* gt, int ldg, void* out,
-                        int ldo, int R, int H, int V, int f32, hipStream_t st) {
+                        int ldo, int R, int H, int V, int per_head, int f32, hipStream_t st) {
   if (R <= 0) return 0;
   dim3 g((H * V + 255) / 256, R), b(256);
   SM_DISPATCH_T(f32, hipLaunchKernelGGL(sigmoid_gate_k<T>, g, b, 0, st, (const T*)o, soh, sor,
-                                         (const T*)gt, ldg, (T*)out, ldo, H, V));
+                                         (const T*)gt, ldg, (T*)out, ldo, H, V, per_head));
   return (int)hipGetLastError();
 }
 

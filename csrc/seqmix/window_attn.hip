@@ -14,9 +14,17 @@
 // window_attn_k: pool row = [k of G heads | v of G heads]; query head h reads key/value head
 // h / (H/G).  Causal sliding window: position i sees j with 0 <= i - j < win.  The softmax
 // denominator holds one more term exp(sink_h) that adds nothing to the numerator: the running
-// maximum starts at sink_h and the running sum at 1 (without a sink: an ordinary softmax).  One block per (query row, key/value head): the
-// heads of the group share the key and value tiles, which stream through LDS with an online
-// softmax.
+// maximum starts at sink_h and the running sum at 1 (without a sink: an ordinary softmax).
+// Optional steps on a score s of query position i and key position j, in this order:
+// cap * tanh(s / cap) (cap > 0), and s - r1_h * ln(1 + r2_h * (i - j)) (r1, r2 given).  Optional
+// head gate: head h of row r leaves multiplied by sigmoid(gate[r, h]).  One block per (query
+// row, key/value head): the heads of the group share the key and value tiles, which stream
+// through LDS with an online softmax.
+//
+// rope_rows_k: turns the channel pairs (2i, 2i+1) of a stretch of every head by pos * inv_freq[i]
+// and writes them to another place (its own rows or scattered ones).  qtemp_kv_store_k: the
+// input pass of attention without rotation: q times the temperature of its position,
+// 1 + coef * ln(floor((p + 1) / every) + 1), to its own buffer, k | v to the token's pool row.
 #include "common.h"
 using namespace sm;
 
@@ -84,6 +92,41 @@ qk_norm_rope_store_k(const T* __restrict__ proj, int ldp, int H, int G, int D, i
     for (int i = threadIdx.x; i < nv; i += blockDim.x) crow[nk + i] = row[nq + nk + i];
 }
 
+template <typename T>
+__global__ void rope_rows_k(const T* __restrict__ src, int lds_, int heads, int src_hs,
+                            const float* __restrict__ inv_freq, int nrot,
+                            const int* __restrict__ pos, const int* __restrict__ out_rows,
+                            T* __restrict__ dst, long ldd, long dst_hs) {
+  const int r = blockIdx.x;
+  const float p = (float)pos[r];
+  const long ro = out_rows ? out_rows[r] : r;
+  if (ro < 0) return;
+  const T* s = src + (size_t)r * lds_;
+  T* d = dst + ro * ldd;
+  for (int idx = threadIdx.x; idx < heads * nrot; idx += blockDim.x) {
+    int h = idx / nrot, i = idx % nrot;
+    float a = ldf(s, (size_t)h * src_hs + 2 * i), b = ldf(s, (size_t)h * src_hs + 2 * i + 1);
+    float sn, cs;
+    sincosf(p * inv_freq[i], &sn, &cs);
+    stf(d, (size_t)(h * dst_hs + 2 * i), a * cs - b * sn);
+    stf(d, (size_t)(h * dst_hs + 2 * i + 1), b * cs + a * sn);
+  }
+}
+
+template <typename T>
+__global__ void qtemp_kv_store_k(const T* __restrict__ proj, int ldp, int nq, int nkv, float coef,
+                                 int every, const int* __restrict__ pos,
+                                 const int* __restrict__ cache_rows, T* __restrict__ pool,
+                                 T* __restrict__ q_out, int ldq) {
+  const int r = blockIdx.x;
+  const T* row = proj + (size_t)r * ldp;
+  const float temp = 1.0f + coef * logf((float)((pos[r] + 1) / every + 1));
+  for (int i = threadIdx.x; i < nq; i += blockDim.x)
+    stf(q_out, (size_t)r * ldq + i, ldf(row, i) * temp);
+  T* crow = pool + (size_t)cache_rows[r] * nkv;
+  for (int i = threadIdx.x; i < nkv; i += blockDim.x) crow[i] = row[nq + i];
+}
+
 #define WA_TK 32       // keys per tile at most
 #define WA_THREADS 256
 #define WA_ACC 16      // (head, value channel) pairs per thread at most
@@ -94,7 +137,8 @@ window_attn_k(const T* __restrict__ q, int ldq, const T* __restrict__ pool,
               const int* __restrict__ bt, int max_pages, const int* __restrict__ row_ent,
               const int* __restrict__ pos, const float* __restrict__ sink, float scale, int win,
               T* __restrict__ out, int ldo, int H, int G, int D, int V, int page, int TK,
-              float out_scale, int HB) {
+              float out_scale, int HB, float cap, const float* __restrict__ r1,
+              const float* __restrict__ r2, const T* __restrict__ gate, int ldg) {
   extern __shared__ float smem[];
   // a block takes up to HB query heads of one key/value head (all of them when they fit)
   const int nhb = (H / G + HB - 1) / HB;
@@ -147,6 +191,8 @@ window_attn_k(const T* __restrict__ q, int ldq, const T* __restrict__ pool,
         float d = 0.0f;
         for (int i = 0; i < D; i++) d += qh[i] * kr[i];
         s = d * scale;
+        if (cap > 0.0f) s = cap * tanhf(s / cap);
+        if (r1) s -= r1[h0 + h] * log1pf(r2[h0 + h] * (float)(p - (j0 + jj)));
       }
       sp[idx] = s;
     }
@@ -187,7 +233,9 @@ window_attn_k(const T* __restrict__ q, int ldq, const T* __restrict__ pool,
     int idx = tid + a * WA_THREADS;
     if (idx < npair) {
       int h = idx / V;
-      stf(out, (size_t)r * ldo + (size_t)h0 * V + idx, acc[a] / sl[h] * out_scale);
+      float o = acc[a] / sl[h] * out_scale;
+      if (gate) o *= sigmoidf_(ldf(gate, (size_t)r * ldg + h0 + h));
+      stf(out, (size_t)r * ldo + (size_t)h0 * V + idx, o);
     }
   }
 }
@@ -208,12 +256,36 @@ int p2p_sm_qk_norm_rope_store(const void* proj, int ldp, int H, int G, int D, in
   return (int)hipGetLastError();
 }
 
+int p2p_sm_rope_rows(const void* src, int lds_, int heads, int src_hs, const float* inv_freq,
+                     int nrot, const int* pos, const int* out_rows, void* dst, long ldd,
+                     long dst_hs, int R, int f32, hipStream_t st) {
+  if (R <= 0 || heads <= 0 || nrot <= 0) return 0;
+  int threads = heads * nrot >= 256 ? 256 : 64;
+  SM_DISPATCH_T(f32, hipLaunchKernelGGL(rope_rows_k<T>, dim3(R), dim3(threads), 0, st,
+                                         (const T*)src, lds_, heads, src_hs, inv_freq, nrot, pos,
+                                         out_rows, (T*)dst, ldd, dst_hs));
+  return (int)hipGetLastError();
+}
+
+int p2p_sm_qtemp_kv_store(const void* proj, int ldp, int nq, int nkv, float coef, int every,
+                          const int* pos, const int* cache_rows, void* pool, void* q_out, int ldq,
+                          int R, int f32, hipStream_t st) {
+  if (R <= 0) return 0;
+  if (nq < 1 || nkv < 1 || every < 1) return (int)hipErrorInvalidValue;
+  SM_DISPATCH_T(f32, hipLaunchKernelGGL(qtemp_kv_store_k<T>, dim3(R), dim3(256), 0, st,
+                                         (const T*)proj, ldp, nq, nkv, coef, every, pos,
+                                         cache_rows, (T*)pool, (T*)q_out, ldq));
+  return (int)hipGetLastError();
+}
+
 int p2p_sm_window_attn(const void* q, int ldq, const void* pool, const int* bt, int max_pages,
                        const int* row_ent, const int* pos, const float* sink, float scale, int win,
                        void* out, int ldo, int R, int H, int G, int D, int V, int page,
-                       float out_scale, int f32, hipStream_t st) {
+                       float out_scale, float cap, const float* r1, const float* r2,
+                       const void* gate, int ldg, int f32, hipStream_t st) {
   if (R <= 0) return 0;
-  if (H < 1 || G < 1 || H % G || D < 1 || V < 1 || win < 1) return (int)hipErrorInvalidValue;
+  if (H < 1 || G < 1 || H % G || D < 1 || V < 1 || win < 1 || (r1 && !r2) || cap < 0.0f)
+    return (int)hipErrorInvalidValue;
   int HG = H / G, TK = WA_TK, HB = HG;
   auto lds = [&](int tk, int hb) {
     return ((size_t)hb * D + (size_t)tk * (D + 1) + (size_t)tk * (V + 1) + (size_t)hb * tk +
@@ -230,7 +302,7 @@ int p2p_sm_window_attn(const void* q, int ldq, const void* pool, const int* bt, 
   SM_DISPATCH_T(f32, hipLaunchKernelGGL(window_attn_k<T>, grid, dim3(WA_THREADS), lds(TK, HB), st,
                                          (const T*)q, ldq, (const T*)pool, bt, max_pages, row_ent,
                                          pos, sink, scale, win, (T*)out, ldo, H, G, D, V, page, TK,
-                                         out_scale, HB));
+                                         out_scale, HB, cap, r1, r2, (const T*)gate, ldg));
   return (int)hipGetLastError();
 }
 

@@ -1,7 +1,9 @@
 // Grouped-query window attention on the matrix cores (bf16 activations, fp32 scores / softmax /
 // sums).  Same inputs and outputs as window_attn_k: pool row = [k of G heads | v of G heads],
 // query head h reads key/value head h / (H/G), causal sliding window of `win` keys, softmax
-// denominator with one more term exp(sink_h).
+// denominator with one more term exp(sink_h); optionally scores capped by cap * tanh(s / cap),
+// a per-head penalty r1_h * ln(1 + r2_h * distance) taken off them, and every head's result
+// multiplied by sigmoid(gate[row, head]).
 //
 // The query heads of one key/value head attend to the same keys, so (row, head) pairs are the M
 // dimension: one wavefront owns 16 pairs -- RW consecutive rows of one sequence portion x HS
@@ -29,7 +31,9 @@ window_attn_mfma_k(const bf16* __restrict__ q, int ldq, const bf16* __restrict__
                    const int* __restrict__ pos, const int* __restrict__ units,
                    const float* __restrict__ sink, float scale, int win, bf16* __restrict__ out,
                    int ldo, int H, int G, int D, int V, int page, int HS, int splits,
-                   float* __restrict__ part, float out_scale) {
+                   float* __restrict__ part, float out_scale, float cap,
+                   const float* __restrict__ r1, const float* __restrict__ r2,
+                   const bf16* __restrict__ gate, int ldg) {
   constexpr int DP = NK * 32;        // padded key size
   constexpr int VP = NV2 * 32;       // padded value size
   constexpr int NT = NV2 * 2;        // 16-wide output column tiles
@@ -72,6 +76,7 @@ window_attn_mfma_k(const bf16* __restrict__ q, int ldq, const bf16* __restrict__
   }
   __syncthreads();
 
+  const float pr1 = (pvalid && r1) ? r1[ph] : 0.0f, pr2 = (pvalid && r1) ? r2[ph] : 0.0f;
   const bool sunk = first && sink != nullptr;   // no sink: an ordinary softmax
   float m_run = pvalid ? (sunk ? sink[ph] : -1e30f) : 0.0f;
   float l_part = (pvalid && quad == 0 && sunk) ? 1.0f : 0.0f;
@@ -129,7 +134,12 @@ window_attn_mfma_k(const bf16* __restrict__ q, int ldq, const bf16* __restrict__
       for (int i = 0; i < 4; i++) {
         int j = j0 + sub * 16 + quad * 4 + i;
         bool ok = pvalid && j <= ppos && j > ppos - win && j <= j_hi;
-        float v = ok ? s[sub][i] * scale : -INFINITY;
+        float v = -INFINITY;
+        if (ok) {
+          v = s[sub][i] * scale;
+          if (cap > 0.0f) v = cap * tanhf(v / cap);
+          if (r1) v -= pr1 * log1pf(pr2 * (float)(ppos - j));
+        }
         sv[sub * 4 + i] = v;
         tmax = fmaxf(tmax, v);
       }
@@ -198,10 +208,12 @@ window_attn_mfma_k(const bf16* __restrict__ q, int ldq, const bf16* __restrict__
     int mr = m / HS, ms = hb0 + m % HS;
     if (mr < nr && ms < HG) {
       bf16* o = out + (size_t)(r0 + mr) * ldo + (size_t)(g * HG + ms) * V;
+      float gv = inv[i];
+      if (gate) gv *= sigmoidf_(__bfloat162float(gate[(size_t)(r0 + mr) * ldg + g * HG + ms]));
 #pragma unroll
       for (int t = 0; t < NT; t++) {
         int c = t * 16 + n16;
-        if (c < V) o[c] = __float2bfloat16(acc[t][i] * inv[i]);
+        if (c < V) o[c] = __float2bfloat16(acc[t][i] * gv);
       }
     }
   }
@@ -211,7 +223,8 @@ window_attn_mfma_k(const bf16* __restrict__ q, int ldq, const bf16* __restrict__
 // One block per (unit, head block, pair); the weights of the runs are formed once in LDS.
 __global__ void window_attn_merge_k(const float* __restrict__ part, const int* __restrict__ units,
                                     bf16* __restrict__ out, int ldo, int H, int G, int V, int HS,
-                                    int splits, int VP, float out_scale) {
+                                    int splits, int VP, float out_scale,
+                                    const bf16* __restrict__ gate, int ldg) {
   __shared__ float sw[65];
   const int r0 = units[2 * blockIdx.x], nr = units[2 * blockIdx.x + 1];
   const int HG = H / G, hblocks = (HG + HS - 1) / HS;
@@ -232,7 +245,10 @@ __global__ void window_attn_merge_k(const float* __restrict__ part, const int* _
     float d = z < splits ? w * rec[z * zs + VP + 1] : 0.0f;
     d = wave_sum(d);
     sw[z] = w;
-    if (z == 0) sw[64] = d > 0.0f ? out_scale / d : 0.0f;
+    if (z == 0) {
+      float gv = gate ? sigmoidf_(__bfloat162float(gate[(size_t)(r0 + mr) * ldg + g * HG + ms])) : 1.0f;
+      sw[64] = d > 0.0f ? out_scale * gv / d : 0.0f;
+    }
   }
   __syncthreads();
   float inv = sw[64];
@@ -268,10 +284,11 @@ int p2p_sm_window_attn_mfma(const void* q, int ldq, const void* pool, const int*
                             int max_pages, const int* row_ent, const int* pos, const int* units,
                             int U, const float* sink, float scale, int win, void* out, int ldo,
                             int H, int G, int D, int V, int page, int splits, float* part,
-                            float out_scale, hipStream_t st) {
+                            float out_scale, float cap, const float* r1, const float* r2,
+                            const void* gate, int ldg, hipStream_t st) {
   if (U <= 0) return 0;
   if (H < 1 || G < 1 || H % G || D < 8 || D > 256 || D % 8 || V < 8 || V > 256 || V % 8 ||
-      win < 1 || ldq % 8)
+      win < 1 || ldq % 8 || (r1 && !r2) || cap < 0.0f)
     return (int)hipErrorInvalidValue;
   if (splits < 1 || splits > 64 || (splits > 1 && !part)) return (int)hipErrorInvalidValue;
   int HG = H / G, HS = head_slots(HG);
@@ -283,11 +300,11 @@ int p2p_sm_window_attn_mfma(const void* q, int ldq, const void* pool, const int*
     hipLaunchKernelGGL((window_attn_mfma_k<NKK, NVV>), grid, block, shm, st, (const bf16*)q,   \
                        ldq, (const bf16*)pool, bt, max_pages, row_ent, pos, units, sink,       \
                        scale, win, (bf16*)out, ldo, H, G, D, V, page, HS, splits, part,        \
-                       out_scale);                                                             \
+                       out_scale, cap, r1, r2, (const bf16*)gate, ldg);                        \
     if (splits > 1)                                                                            \
       hipLaunchKernelGGL(window_attn_merge_k, dim3(grid.x, grid.y, 16), dim3(128), 0, st,      \
                          part, units, (bf16*)out, ldo, H, G, V, HS, splits, NVV * 32,          \
-                         out_scale);                                                           \
+                         out_scale, (const bf16*)gate, ldg);                                   \
   } while (0)
 #define WMV(NKK)                 \
   do {                           \

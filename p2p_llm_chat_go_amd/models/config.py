@@ -123,6 +123,13 @@ def _hybrid_presets() -> dict:
     gelu = {"kind": "dense", "ff": 512}
     smoe = {"kind": "moe", "expert": {"ff": 128}, "shared": {"ff": 256},
             "router": {"experts": 6, "identity": 2, "top": 2, "groups": {"count": 4, "keep": 2}}}
+    ba = {"type": "attention",
+          "mixer": {"heads": 8, "kv_heads": 2, "dim": 32, "vdim": 32, "scale": 32 ** -0.5, "softcap": 30.0,
+                    "q_temp": {"coef": 0.1, "every": 128}}}
+    rl = {"type": "latent_attention",
+          "mixer": {"heads": 4, "dim": 32, "rot_dim": 16, "vdim": 32, "kv_rank": 64, "q_rank": 96,
+                    "rot": {"base": 10000.0, "dims": 16}, "scale": 48 ** -0.5}}
+    tmoe = {"kind": "moe", "expert": {"ff": 128}, "shared": {"ff": 256}, "router": {"experts": 8, "top": 2}}
     return {"tiny-regesun": HybridConfig.from_dict(
         {"architecture": "Regesun", "width": 256, "vocab": 512, "max_positions": 4096,
          "norm": {"eps": 1e-5}, "layers": [gd, mb, la, mb, gd, la], "eos_token_id": [2]},
@@ -135,12 +142,18 @@ def _hybrid_presets() -> dict:
         {"architecture": "Futetar", "width": 256, "vocab": 512, "norm": {"eps": 1e-6},
          "layers": [dict(at, mlp=gelu), dict(ml, mlp=smoe), dict(ml, mlp=gelu),
                     {"type": "attention", "mixer": dict(at["mixer"], kv_from=0), "mlp": smoe}, ml],
-         "eos_token_id": [2]}, name="tiny-futetar")}
+         "eos_token_id": [2]}, name="tiny-futetar"),
+        "tiny-tarunex": HybridConfig.from_dict(
+        {"architecture": "Tarunex", "width": 256, "vocab": 512, "norm": {"eps": 1e-5},
+         "embedding": {"scale": 16.0}, "logit_scale": 0.5, "logit_softcap": 30.0,
+         "loop": {"start": 1, "stop": 3, "times": 2},
+         "layers": [dict(ba, mlp=tmoe), dict(rl, mlp=tmoe), dict(ba, mlp=tmoe), dict(rl, mlp=None)],
+         "eos_token_id": [2]}, name="tiny-tarunex")}
 
 
 def get_config(name: str):
     key = ALIASES.get(name, name)
-    if key not in PRESETS and key.endswith(("regesun", "rotutar", "futetar")):
+    if key not in PRESETS and key.endswith(("regesun", "rotutar", "futetar", "tarunex")):
         hp = _hybrid_presets()
         if key in hp:
             return hp[key]

@@ -1264,7 +1264,9 @@ def random_state_dict(cfg: HybridConfig, seed: int = 0) -> dict:
     step parameters in the ranges where the recurrences neither vanish nor blow up."""
     g = torch.Generator().manual_seed(seed)
     sd = {}
-    for k, s in tensor_shapes(cfg).items():
+    shapes = tensor_shapes(cfg)
+    for k, s in shapes.items():
+        s = tuple(s) or (1,)   # a single number is drawn as one and stored without a shape
         leaf = k.split(".", 1)[1] if k.startswith("l") and "." in k else k
         if len(s) == 2 and not leaf.endswith("conv"):
             t = torch.randn(*s, generator=g) / (s[1] ** 0.5 if k not in ("embed", "pos") else 1.0)
@@ -1290,7 +1292,7 @@ def random_state_dict(cfg: HybridConfig, seed: int = 0) -> dict:
             t = torch.randn(*s, generator=g) * 0.5
         else:
             t = torch.randn(*s, generator=g) * 0.5
-        sd[k] = t.to(torch.bfloat16)
+        sd[k] = t.to(torch.bfloat16).reshape(tuple(shapes[k]))
     return sd
 
 

@@ -68,12 +68,13 @@ def parse(argv=None):
                     help="cpu: gloo + the CPU engine (plumbing tests with tiny models)")
     ap.add_argument("--hybrid", action="store_true",
                     help="instead of the headline workload: prefill / decode throughput of "
-                         "hybrid models (Regesun, Rotutar, Futetar) beside a dense Llama of equal size "
+                         "hybrid models (Regesun, Rotutar, Futetar, Tarunex) beside a dense Llama of equal size "
                          "(bench/hybrid_bench.py; 1 GPU)")
-    ap.add_argument("--hybrid-design", choices=("regesun", "rotutar", "futetar", "both"),
+    ap.add_argument("--hybrid-design", choices=("regesun", "rotutar", "futetar", "tarunex", "both"),
                     default="regesun",
                     help="regesun: Regesun beside the Llama; rotutar: Rotutar beside Regesun "
-                         "(equal width and depth); futetar: Futetar beside Rotutar; both: "
+                         "(equal width and depth); futetar: Futetar beside Rotutar; tarunex: Tarunex "
+                         "beside Futetar; both: "
                          "Rotutar, Regesun and the Llama")
     ap.add_argument("--hybrid-phase", choices=("both", "prefill", "decode"), default="both",
                     help="measure only the prompt or only the decode workload (profiling)")

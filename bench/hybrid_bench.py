@@ -1,13 +1,15 @@
-"""Prefill and decode throughput of hybrid models (Regesun, Rotutar, Futetar) at layer sizes that
+"""Prefill and decode throughput of hybrid models (Regesun, Rotutar, Futetar, Tarunex) at layer sizes that
 resemble real models, beside a dense Llama of the same width, depth and parameter count on
 the same engine entry point (``generate``).  Random weights, random tokens.
 
-    python bench.py --hybrid [--hybrid-design regesun|rotutar|futetar|both] [--hybrid-sizes 1024,2048]
+    python bench.py --hybrid [--hybrid-design regesun|rotutar|futetar|tarunex|both] [--hybrid-sizes 1024,2048]
                     [--steps K] [--warmup W]
 
 ``--hybrid-design rotutar`` runs Rotutar beside Regesun (the closest model: same engine, same
 width and depth) instead of the Llama; ``futetar`` runs Futetar beside Rotutar (gated scans,
-grouped-query attention and routed experts in both).
+grouped-query attention and routed experts in both); ``tarunex`` runs Tarunex beside Futetar
+(parallel layers, grouped-query attention and routed experts with a shared expert in both; 16
+layer runs each).
 
 One JSON line per (size, model): prefill tokens/s of one long prompt (``prompt`` tokens),
 decode tokens/s of ``batch`` sequences.  These lines are not the headline metric.
@@ -85,6 +87,29 @@ def futetar_config(width: int):
          "layers": layers}, name="futetar-w%d" % width)
 
 
+def tarunex_config(width: int):
+    """A Tarunex stack at a given width: 10 layers of which the middle 6 run two passes (16 layer
+    runs), biased attention three times for every latent attention, every layer with routed
+    experts and a shared expert, 128-wide heads."""
+    from p2p_llm_chat_go_amd.models.hybrid import HybridConfig
+
+    hd = 128
+    nh = width // hd
+    moe = {"kind": "moe", "expert": {"ff": width // 2}, "shared": {"ff": width // 2},
+           "router": {"experts": 8, "top": 2}}
+    ba = {"type": "attention",
+          "mixer": {"heads": nh, "kv_heads": max(1, nh // 4), "dim": hd, "vdim": hd, "scale": hd ** -0.5,
+                    "softcap": 30.0, "q_temp": {"coef": 0.1, "every": 512}}, "mlp": moe}
+    la = {"type": "latent_attention",
+          "mixer": {"heads": nh, "dim": hd, "rot_dim": 64, "vdim": hd, "kv_rank": 448, "q_rank": width // 2,
+                    "rot": {"base": 10000.0, "dims": 64}, "scale": (hd + 64) ** -0.5}, "mlp": moe}
+    layers = [ba, ba, ba, la, ba, ba, la, ba, ba, la]
+    return HybridConfig.from_dict(
+        {"architecture": "Tarunex", "width": width, "vocab": 32000, "norm": {"eps": 1e-5},
+         "embedding": {"scale": width ** 0.5}, "logit_scale": 0.25, "logit_softcap": 30.0,
+         "loop": {"start": 2, "stop": 8, "times": 2}, "layers": layers}, name="tarunex-w%d" % width)
+
+
 def n_params(cfg) -> int:
     from p2p_llm_chat_go_amd.models.hybrid import tensor_shapes
 
@@ -153,6 +178,7 @@ def run(a):
         lcfg = llama_like(width, hcfg.n_layers, params)
         todo = {"regesun": lambda: (hcfg, lcfg), "rotutar": lambda: (rotutar_config(width), hcfg),
                 "futetar": lambda: (futetar_config(width), rotutar_config(width)),
+                "tarunex": lambda: (tarunex_config(width), futetar_config(width)),
                 "both": lambda: (rotutar_config(width), hcfg, lcfg)}[design]()
         for cfg in todo:
             if getattr(a, "hybrid_only", None) and a.hybrid_only not in cfg.name:
@@ -171,7 +197,8 @@ def run(a):
                         getattr(a, "hybrid_phase", "both"))
             line = {"metric": "hybrid-vs-dense throughput", "model": cfg.name,
                     "params_m": round((params if hybrid else cfg.n_params()) / 1e6, 1),
-                    "width": width, "layers": cfg.n_layers, "dtype": "bf16",
+                    "width": width, "layers": cfg.n_layers,
+                    "layer_runs": len(cfg.runs()) if hybrid else cfg.n_layers, "dtype": "bf16",
                     "prompt_tokens": prompt, "decode_batch": batch, "decode_ctx": ctx,
                     "new_tokens": new, "steps": a.steps, "warmup": a.warmup,
                     "data": "random tokens; random-init weights",

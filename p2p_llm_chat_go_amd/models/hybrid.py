@@ -10,6 +10,10 @@ is wrapped around the residual stream,
                                                              equal parts of the vector
     "parallel"    x <- x + mixer(u) + ff(u),  u = norm(x)    one norm per layer feeds both
                                                              sublayers
+    "parallel2"   x <- x + mixer(norm1(x)) + ff(norm2(x))    a norm per sublayer, each with
+                                                             one weight for all channels; a
+                                                             stretch of layers may run several
+                                                             passes (``loop``)
 
 and whether learned absolute positions are added to the token embedding.  Mixers:
 
@@ -32,17 +36,30 @@ and whether learned absolute positions are added to the token embedding.  Mixers
                         positions on channel pairs (i, i + dims/2) with optional stretching of
                         the long wavelengths; a layer may read an earlier layer's keys and
                         values (``kv_from``) instead of projecting its own;
+  ``biased_attention``  causal grouped-query attention without rotation: biased projections, a
+                        query temperature that grows with the logarithm of the position, capped
+                        scores, a logarithmic distance penalty per head, a softmax sink with
+                        score 0, one sigmoid gate per head;
+  ``rope_latent_attention``  latent attention with low-rank queries and one rotated key part
+                        that the heads share, cached beside the latent; plain causal softmax, one
+                        sigmoid gate per head;
   ``parallel``          two mixers side by side on the same input, summed with fixed scales.
 
 Feed-forwards: ``dense`` (silu-gated, or the clamped gated unit when the config gives a
-limit) and ``moe`` (sigmoid router, choice limited to the best groups of experts).
+limit), ``moe`` (sigmoid router, choice limited to the best groups of experts), ``moe_softmax``
+and ``moe_top`` (biased router, softmax over the chosen logits, silu-gated experts, shared expert).
+A design may give a config's ``type`` / ``kind`` names a meaning of its own (``Design.mixers``,
+``Design.ff``).
 
 "Regesun" stacks the first three mixers in the sandwich form with learned positions;
 "Rotutar" stacks ``parallel`` (window attention beside the gated delta rule) and ``hgrn2``
 layers in the gated post-norm form, without positions other than the rotation, and caps
 its logits with a tanh.  "Futetar" stacks ``mlstm`` and ``attention`` layers in the parallel
 form (norm weights stored around zero), with gelu-gated dense feed-forwards and mixtures of
-squared-relu experts behind a softmax router.  A checkpoint is a ``config.json`` whose
+squared-relu experts behind a softmax router.  "Tarunex" stacks ``biased_attention`` and
+``rope_latent_attention`` layers (its config calls them "attention" and "latent_attention") in
+the two-norm parallel form with ``moe_top`` feed-forwards, repeats a stretch of layers, scales
+its embedding and scales and caps its logits.  A checkpoint is a ``config.json`` whose
 ``architecture`` names the design and one safetensors file (``load_dir``).
 
 One ``forward`` serves every step: a flat list of token rows cut into entries (portions of

@@ -13,7 +13,9 @@ STRICT_SENDER, UI_FILE) and the engine knobs:
                   tiny-rotutar: a small hybrid of window attention beside a gated delta
                   rule, HGRN2 layers and a group-limited mixture of experts;
                   tiny-futetar: a small hybrid of mLSTM and attention layers with
-                  softmax-routed experts)
+                  softmax-routed experts;
+                  tiny-tarunex: a small attention-only model with repeated layers,
+                  biased and latent attention and top-routed experts)
   ENGINE_DEVICE   cuda:N / cpu (default: cuda:0 if available)
   ENGINE_CHECKPOINT  checkpoint dir (safetensors + config.json: HF Llama / Mixtral, or a
                   hybrid design named by its "architecture" key); default random-init

@@ -193,8 +193,9 @@ __global__ void add_norm_k(float* __restrict__ x, const T* __restrict__ a, int l
     stf(h, (size_t)r * ldh + i, xr[i] * r2 * w2[i]);
 }
 
-// x += a + b + rows + vec on the fp32 residual (each addend optional; a, b activation typed,
-// rows fp32 [R, n], vec fp32 [n]; summed first, in fp32), then up to two normed copies of the
+// x += a + b + rows + vec + sum_k cw[r, k] * cy[r * top + k] on the fp32 residual (each addend
+// optional; a, b, cy activation typed, rows fp32 [R, n], vec fp32 [n], cw fp32 [R, top]: the
+// weighted sum of a token's routed expert outputs; summed first, in fp32), then up to two normed copies of the
 // updated row, h_i = x / sqrt(mean(x^2) + eps) * w_i, where w_i is a vector (ws_i = 1) or one
 // number for all channels (ws_i = 0): two sublayers that read the same row through norms of
 // their own get their inputs from one pass over it.
@@ -203,33 +204,74 @@ __global__ void add_norm2_k(float* __restrict__ x, const T* __restrict__ a, int 
                             const T* __restrict__ b, int ldb, const float* __restrict__ rows,
                             const float* __restrict__ vec, int n, float eps,
                             const float* __restrict__ w1, int ws1, T* __restrict__ h1, int ld1,
-                            const float* __restrict__ w2, int ws2, T* __restrict__ h2, int ld2) {
+                            const float* __restrict__ w2, int ws2, T* __restrict__ h2, int ld2,
+                            const T* __restrict__ cy, int ldcy, const float* __restrict__ cw,
+                            int top) {
   __shared__ float red[16];
   int r = blockIdx.x;
+  const T* cyr = cy ? cy + (size_t)r * top * ldcy : nullptr;
+  const float* cwr = cy ? cw + (size_t)r * top : nullptr;
   const T* ar = a ? a + (size_t)r * lda : nullptr;
   const T* br = b ? b + (size_t)r * ldb : nullptr;
   const float* er = rows ? rows + (size_t)r * n : nullptr;
   float* xr = x + (size_t)r * n;
-  const bool adds = ar || br || er || vec;
+  const bool adds = ar || br || er || vec || cyr;
+  // weights that are one number are read before the reduction
+  const float g1 = (w1 && !ws1) ? w1[0] : 1.0f, g2 = (w2 && !ws2) ? w2[0] : 1.0f;
   if (n <= NV * (int)blockDim.x) {
-    // every load goes out before the first store
-    float xv[NV];
+    // every load goes out before the first store; each addend's loads form one batch (the
+    // tests for the optional addends stay outside the unrolled loops)
+    float xv[NV], yv[NV];
     float s2 = 0.0f;
 #pragma unroll
     for (int k = 0; k < NV; k++) {
       int i = threadIdx.x + k * blockDim.x;
-      bool ok = i < n;
-      int ic = ok ? i : 0;
-      float y = 0.0f;
-      if (ar) y += ldf(ar, ic);
-      if (br) y += ldf(br, ic);
-      if (er) y += er[ic];
-      if (vec) y += vec[ic];
-      xv[k] = ok ? xr[ic] + y : 0.0f;
+      xv[k] = xr[i < n ? i : 0];
+      yv[k] = 0.0f;
+    }
+    if (ar) {
+#pragma unroll
+      for (int k = 0; k < NV; k++) {
+        int i = threadIdx.x + k * blockDim.x;
+        yv[k] = ldf(ar, i < n ? i : 0);
+      }
+    }
+    if (br) {
+#pragma unroll
+      for (int k = 0; k < NV; k++) {
+        int i = threadIdx.x + k * blockDim.x;
+        yv[k] += ldf(br, i < n ? i : 0);
+      }
+    }
+    if (er) {
+#pragma unroll
+      for (int k = 0; k < NV; k++) {
+        int i = threadIdx.x + k * blockDim.x;
+        yv[k] += er[i < n ? i : 0];
+      }
+    }
+    if (vec) {
+#pragma unroll
+      for (int k = 0; k < NV; k++) {
+        int i = threadIdx.x + k * blockDim.x;
+        yv[k] += vec[i < n ? i : 0];
+      }
+    }
+    if (cyr) {
+      for (int t = 0; t < top; t++) {
+        const float wt = cwr[t];
+        const T* yr = cyr + (size_t)t * ldcy;
+#pragma unroll
+        for (int k = 0; k < NV; k++) {
+          int i = threadIdx.x + k * blockDim.x;
+          yv[k] += wt * ldf(yr, i < n ? i : 0);
+        }
+      }
     }
 #pragma unroll
     for (int k = 0; k < NV; k++) {
       int i = threadIdx.x + k * blockDim.x;
+      xv[k] = i < n ? xv[k] + yv[k] : 0.0f;
       if (adds && i < n) xr[i] = xv[k];
       s2 += xv[k] * xv[k];
     }
@@ -240,8 +282,9 @@ __global__ void add_norm2_k(float* __restrict__ x, const T* __restrict__ a, int 
     for (int k = 0; k < NV; k++) {
       int i = threadIdx.x + k * blockDim.x;
       if (i < n) {
-        stf(h1, (size_t)r * ld1 + i, xv[k] * r2 * w1[ws1 ? i : 0]);
-        if (w2) stf(h2, (size_t)r * ld2 + i, xv[k] * r2 * w2[ws2 ? i : 0]);
+        float v = xv[k] * r2;
+        stf(h1, (size_t)r * ld1 + i, v * (ws1 ? w1[i] : g1));
+        if (w2) stf(h2, (size_t)r * ld2 + i, v * (ws2 ? w2[i] : g2));
       }
     }
     return;
@@ -253,6 +296,8 @@ __global__ void add_norm2_k(float* __restrict__ x, const T* __restrict__ a, int 
     if (br) y += ldf(br, i);
     if (er) y += er[i];
     if (vec) y += vec[i];
+    if (cyr)
+      for (int t = 0; t < top; t++) y += cwr[t] * ldf(cyr, (size_t)t * ldcy + i);
     float v = xr[i] + y;
     if (adds) xr[i] = v;
     s2 += v * v;
@@ -261,9 +306,9 @@ __global__ void add_norm2_k(float* __restrict__ x, const T* __restrict__ a, int 
   s2 = block_sum(s2, red);
   float r2 = 1.0f / sqrtf(s2 / (float)n + eps);
   for (int i = threadIdx.x; i < n; i += blockDim.x) {   // each thread re-reads its own writes
-    float v = xr[i];
-    stf(h1, (size_t)r * ld1 + i, v * r2 * w1[ws1 ? i : 0]);
-    if (w2) stf(h2, (size_t)r * ld2 + i, v * r2 * w2[ws2 ? i : 0]);
+    float v = xr[i] * r2;
+    stf(h1, (size_t)r * ld1 + i, v * (ws1 ? w1[i] : g1));
+    if (w2) stf(h2, (size_t)r * ld2 + i, v * (ws2 ? w2[i] : g2));
   }
 }
 
@@ -398,12 +443,15 @@ int p2p_sm_norm_scale_add(float* x, const void* y, int ldy, const float* w, cons
 
 int p2p_sm_add_norm2(float* x, const void* a, int lda, const void* b, int ldb, const float* rows,
                      const float* vec, int R, int n, float eps, const float* w1, int ws1, void* h1,
-                     int ld1, const float* w2, int ws2, void* h2, int ld2, int f32, hipStream_t st) {
+                     int ld1, const float* w2, int ws2, void* h2, int ld2, const void* cy, int ldcy,
+                     const float* cw, int top, int f32, hipStream_t st) {
   if (R <= 0) return 0;
-  if ((w1 && !h1) || (w2 && (!h2 || !w1)) || (b && !a)) return (int)hipErrorInvalidValue;
+  if ((w1 && !h1) || (w2 && (!h2 || !w1)) || (b && !a) || (cy && (!cw || top < 1)))
+    return (int)hipErrorInvalidValue;
   SM_DISPATCH_T(f32, hipLaunchKernelGGL(add_norm2_k<T>, dim3(R), dim3(256), 0, st, x, (const T*)a,
                                          lda, (const T*)b, ldb, rows, vec, n, eps, w1, ws1,
-                                         (T*)h1, ld1, w2, ws2, (T*)h2, ld2));
+                                         (T*)h1, ld1, w2, ws2, (T*)h2, ld2, (const T*)cy, ldcy,
+                                         cw, top));
   return (int)hipGetLastError();
 }
 

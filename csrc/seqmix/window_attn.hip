@@ -113,6 +113,50 @@ __global__ void rope_rows_k(const T* __restrict__ src, int lds_, int heads, int 
   }
 }
 
+// Input pass of latent attention with low-rank queries: one projection row holds the query
+// latent (nq numbers), the key/value latent (nc) and a key part to be rotated (2 * nrot and what
+// follows it up to nr channels, unrotated).  Both latents are RMS-normalised by themselves and
+// weighted; the query latent goes to its own buffer, the key/value latent and the rotated part
+// to the token's row of the paged pool ([nc | nr]).  Wavefront 0 takes the query latent,
+// wavefront 1 the key/value latent, wavefront 2 the rotation.
+template <typename T>
+__global__ void __launch_bounds__(192)
+latent_prep_k(const T* __restrict__ proj, int ldp, int nq, int nc, int nr,
+              const float* __restrict__ qw, const float* __restrict__ cw,
+              const float* __restrict__ inv_freq, int nrot, const int* __restrict__ pos,
+              const int* __restrict__ cache_rows, T* __restrict__ pool, float eps,
+              T* __restrict__ cq, int ldq) {
+  const int r = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const T* row = proj + (size_t)r * ldp;
+  T* crow = pool + (size_t)cache_rows[r] * (nc + nr);
+  if (wave < 2) {
+    const T* src = row + (wave ? nq : 0);
+    const int n = wave ? nc : nq;
+    const float* w = wave ? cw : qw;
+    T* dst = wave ? crow : cq + (size_t)r * ldq;
+    float ss = 0.0f;
+    for (int i = lane; i < n; i += 64) {
+      float v = ldf(src, i);
+      ss += v * v;
+    }
+    ss = wave_sum(ss);
+    const float rs = 1.0f / sqrtf(ss / (float)n + eps);
+    for (int i = lane; i < n; i += 64) stf(dst, i, ldf(src, i) * rs * w[i]);
+    return;
+  }
+  const T* src = row + nq + nc;
+  T* dst = crow + nc;
+  const float p = (float)pos[r];
+  for (int i = lane; i < nrot; i += 64) {
+    float a = ldf(src, 2 * i), b = ldf(src, 2 * i + 1);
+    float sn, cs;
+    sincosf(p * inv_freq[i], &sn, &cs);
+    stf(dst, 2 * i, a * cs - b * sn);
+    stf(dst, 2 * i + 1, b * cs + a * sn);
+  }
+  for (int i = 2 * nrot + lane; i < nr; i += 64) dst[i] = src[i];
+}
+
 template <typename T>
 __global__ void qtemp_kv_store_k(const T* __restrict__ proj, int ldp, int nq, int nkv, float coef,
                                  int every, const int* __restrict__ pos,
@@ -264,6 +308,18 @@ int p2p_sm_rope_rows(const void* src, int lds_, int heads, int src_hs, const flo
   SM_DISPATCH_T(f32, hipLaunchKernelGGL(rope_rows_k<T>, dim3(R), dim3(threads), 0, st,
                                          (const T*)src, lds_, heads, src_hs, inv_freq, nrot, pos,
                                          out_rows, (T*)dst, ldd, dst_hs));
+  return (int)hipGetLastError();
+}
+
+int p2p_sm_latent_prep(const void* proj, int ldp, int nq, int nc, int nr, const float* qw,
+                       const float* cw, const float* inv_freq, int nrot, const int* pos,
+                       const int* cache_rows, void* pool, float eps, void* cq, int ldq, int R,
+                       int f32, hipStream_t st) {
+  if (R <= 0) return 0;
+  if (nq < 1 || nc < 1 || nr < 0 || nrot < 0 || 2 * nrot > nr) return (int)hipErrorInvalidValue;
+  SM_DISPATCH_T(f32, hipLaunchKernelGGL(latent_prep_k<T>, dim3(R), dim3(192), 0, st,
+                                         (const T*)proj, ldp, nq, nc, nr, qw, cw, inv_freq, nrot,
+                                         pos, cache_rows, (T*)pool, eps, (T*)cq, ldq));
   return (int)hipGetLastError();
 }
 

@@ -22,6 +22,14 @@ using namespace sm;
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
+// cap * tanh(v / cap) and ln(1 + x) on the hardware's exp2 / log2 / reciprocal units: a prompt
+// evaluates them once per (query, key, head), where the library forms (tanhf, log1pf) cost more
+// than the matrix products; their error is far below the bf16 rounding of the probabilities.
+__device__ __forceinline__ float fast_tanh(float x) {
+  float t = __expf(2.0f * x);                       // inf for large x -> 1, 0 for small x -> -1
+  return 1.0f - 2.0f * __frcp_rn(t + 1.0f);
+}
+
 #define WM_LDK 36   // keys per transposed value row in LDS (32 + padding), in bf16
 
 template <int NK, int NV2>  // D padded to NK * 32, V padded to NV2 * 32
@@ -77,6 +85,7 @@ window_attn_mfma_k(const bf16* __restrict__ q, int ldq, const bf16* __restrict__
   __syncthreads();
 
   const float pr1 = (pvalid && r1) ? r1[ph] : 0.0f, pr2 = (pvalid && r1) ? r2[ph] : 0.0f;
+  const float inv_cap = cap > 0.0f ? 1.0f / cap : 0.0f;
   const bool sunk = first && sink != nullptr;   // no sink: an ordinary softmax
   float m_run = pvalid ? (sunk ? sink[ph] : -1e30f) : 0.0f;
   float l_part = (pvalid && quad == 0 && sunk) ? 1.0f : 0.0f;
@@ -137,8 +146,8 @@ window_attn_mfma_k(const bf16* __restrict__ q, int ldq, const bf16* __restrict__
         float v = -INFINITY;
         if (ok) {
           v = s[sub][i] * scale;
-          if (cap > 0.0f) v = cap * tanhf(v / cap);
-          if (r1) v -= pr1 * log1pf(pr2 * (float)(ppos - j));
+          if (cap > 0.0f) v = cap * fast_tanh(v * inv_cap);
+          if (r1) v -= pr1 * __logf(1.0f + pr2 * (float)(ppos - j));
         }
         sv[sub * 4 + i] = v;
         tmax = fmaxf(tmax, v);

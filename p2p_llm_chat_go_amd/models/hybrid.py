@@ -668,14 +668,10 @@ class RopeLatentAttention(Mixer):
         R, dev, dt = b.R, proj.device, proj.dtype
         pool = cache.paged[layer]
         cq = torch.empty(R, qr, device=dev, dtype=dt)
-        sm.rmsnorm(proj[:, :qr], self.qnorm, self.eps, cq)
+        sm.latent_prep(proj, qr, r, Rd, self.qnorm, self.cnorm, self.inv_freq, b.pos, b.cache_rows,
+                       pool, self.eps, cq)
         q = F.linear(cq, self.uq)                                                  # [R, H*(D+Rd)]
-        sm.rmsnorm(proj[:, qr:qr + r], self.cnorm, self.eps, pool[:, :r], out_rows=b.cache_rows)
         nrot2 = self.rot_dims
-        kr = proj[:, qr + r:qr + r + Rd]
-        sm.rope_rows(kr, 1, 0, self.inv_freq, b.pos, pool[:, r:], 0, out_rows=b.cache_rows)
-        if nrot2 < Rd:   # channels of the shared key part beyond the rotated ones pass unchanged
-            pool[b.cache_rows.long(), r + nrot2:] = kr[:, nrot2:]
         qa = torch.empty(H, R, r + Rd, device=dev, dtype=dt)
         q3 = q.view(R, H, D + Rd)
         torch.bmm(q3[:, :, :D].transpose(0, 1), self.uk, out=qa[:, :, :r])
@@ -1095,13 +1091,19 @@ class TopMoEFF:
             self.w_in = torch.cat([get("shared.gate"), get("shared.up")], 0).to(dev, dtype).contiguous()
             self.w_out = get("shared.down").to(dev, dtype).contiguous()
 
-    def routed(self, h):
+    def routed(self, h, cnt=None):
+        """(y [R * top, width], wts [R, top]): the chosen experts' outputs and their weights,
+        to be summed by whoever adds them to the residual.  cnt: cleared int32 counts [E] (a
+        model hands every layer a row of one buffer that it clears once per step)."""
         R, top, dev = h.shape[0], self.top, h.device
         ids = torch.empty(R, top, device=dev, dtype=torch.int32)
         wts = torch.empty(R, top, device=dev, dtype=torch.float32)
-        cnt = torch.empty(self.E, device=dev, dtype=torch.int32)
+        cleared = cnt is not None
+        if cnt is None:
+            cnt = torch.empty(self.E, device=dev, dtype=torch.int32)
         rows = torch.empty(self.E, R * top, device=dev, dtype=torch.int32)
-        sm.group_route(h, self.wr, top, 1, 1, ids, wts, cnt, rows, score="top_softmax", bias=self.br)
+        sm.group_route(h, self.wr, top, 1, 1, ids, wts, cnt, rows, score="top_softmax", bias=self.br,
+                       cleared=cleared)
         act = torch.empty(R * top, self.F, device=dev, dtype=h.dtype)
         if self.fused:
             sm.expert_gemm(h, top, self.w_gu, cnt, rows, act, R * top, silu_glu=True)
@@ -1111,16 +1113,21 @@ class TopMoEFF:
             sm.glu_act(gu, act, "silu")
         y = torch.empty(R * top, self.width, device=dev, dtype=h.dtype)
         sm.expert_gemm(act, 1, self.w_down, cnt, rows, y, R * top)
-        out = torch.empty(R, self.width, device=dev, dtype=h.dtype)
-        return sm.expert_combine(y, wts, out)
+        return y, wts
 
-    def fill(self, proj, h, mid):
+    def fill_routed(self, proj, h, mid, cnt=None):
+        """``fill`` for a layer whose residual pass sums the routed experts itself."""
         if self.Fs:
             sm.glu_act(proj, mid, "silu")
-        return self.routed(h)
+        return self.routed(h, cnt)
+
+    def fill(self, proj, h, mid):
+        y, wts = self.fill_routed(proj, h, mid)
+        return sm.expert_combine(y, wts, torch.empty(h.shape[0], self.width, device=h.device, dtype=h.dtype))
 
     def forward(self, h):
-        y = self.routed(h)
+        y, wts = self.routed(h)
+        y = sm.expert_combine(y, wts, torch.empty(h.shape[0], self.width, device=h.device, dtype=h.dtype))
         if self.Fs:
             mid = torch.empty(h.shape[0], self.Fs, device=h.device, dtype=h.dtype)
             sm.glu_act(F.linear(h, self.w_in), mid, "silu")
@@ -1390,26 +1397,33 @@ class HybridModel:
         h1 = torch.empty(R, W, device=self.device, dtype=self.dtype)
         h2 = torch.empty(R, W, device=self.device, dtype=self.dtype)
         runs = cfg.runs()
-        y = extra = None   # what the previous layer adds to x
+        # the experts' slot counts of all layer runs, cleared by one fill
+        moe = [hasattr(w.layers[i].ff, "fill_routed") for i, _t, _f in runs]
+        cnts = torch.zeros(sum(moe), max([w.layers[i].ff.E for (i, _t, _f), m in zip(runs, moe) if m] or [1]),
+                           device=self.device, dtype=torch.int32) if any(moe) else None
+        y = extra = routed = None   # what the previous layer adds to x
         for k, (i, t, first) in enumerate(runs):
             L = w.layers[i]
             n2, o2 = (L.norm2, h2) if L.ff is not None else (None, None)
             if layer_out is not None and y is not None:   # the rows between two layers are asked for
-                sm.add_norm2(x, y, extra)
+                sm.add_norm2(x, y, extra, routed=routed)
                 layer_out.append(x.clone())
-                y = extra = None
+                y = extra = routed = None
             sm.add_norm2(x, y, extra, rows=x0 if first and t > 0 else None,
                          vec=w.loop_step[t] if first else None, eps=cfg.eps,
-                         w1=L.norm1, out1=h1, w2=n2, out2=o2)
+                         w1=L.norm1, out1=h1, w2=n2, out2=o2, routed=routed)
             mm = L.mixer.n_mid
             mid = torch.empty(R, L.w_out_all.shape[1], device=self.device, dtype=self.dtype)
             L.mixer.mix(F.linear(h1, L.mixer.w_in, L.mixer.b_in), b, self.cache, k, mid[:, :mm])
-            extra = None
+            extra = routed = None
             if L.ff is not None:
                 proj = F.linear(h2, L.ff.w_in) if L.ff.w_in is not None else None
-                extra = L.ff.fill(proj, h2, mid[:, mm:])
+                if moe[k]:
+                    routed = L.ff.fill_routed(proj, h2, mid[:, mm:], cnts[sum(moe[:k]), :L.ff.E])
+                else:
+                    extra = L.ff.fill(proj, h2, mid[:, mm:])
             y = F.linear(mid, L.w_out_all)
-        sm.add_norm2(x, y, extra)
+        sm.add_norm2(x, y, extra, routed=routed)
         if layer_out is not None:
             layer_out.append(x.clone())
         if b.n_out == 0:

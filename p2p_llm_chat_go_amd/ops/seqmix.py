@@ -76,7 +76,10 @@ _SIGS = {
                         c_void_p, c_void_p, c_int, c_int, c_void_p],
     "p2p_sm_add_norm2": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int,
                          c_int, c_float, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int,
-                         c_void_p, c_int, c_int, c_void_p],
+                         c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p],
+    "p2p_sm_latent_prep": [c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p,
+                           c_int, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_int, c_int,
+                           c_int, c_void_p],
     "p2p_sm_rope_rows": [c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p,
                          c_void_p, c_long, c_long, c_int, c_int, c_void_p],
     "p2p_sm_qtemp_kv_store": [c_void_p, c_int, c_int, c_int, c_float, c_int, c_void_p, c_void_p,
@@ -338,10 +341,11 @@ def add_norm(x, a, b=None, eps: float = 0.0, next_w=None, next_out=None):
 
 
 def add_norm2(x, a=None, b=None, rows=None, vec=None, eps: float = 0.0, w1=None, out1=None,
-              w2=None, out2=None):
-    """x += a + b + rows + vec on the fp32 residual x (every addend optional; a, b activation
-    typed [R, n], rows fp32 [R, n], vec fp32 [n]; they are summed in fp32 before they meet x),
-    then up to two normed copies of the updated rows in the same pass,
+              w2=None, out2=None, routed=None):
+    """x += a + b + rows + vec + routed on the fp32 residual x (every addend optional; a, b
+    activation typed [R, n], rows fp32 [R, n], vec fp32 [n]; routed = (y, wts): the weighted
+    sum over a token's routed experts, sum_k wts[r, k] * y[r * top + k], y activation typed
+    [R * top, n], wts fp32 [R, top]; they are summed in fp32 before they meet x), then up to two normed copies of the updated rows in the same pass,
     out_i = x / sqrt(mean(x^2) + eps) * w_i, each w_i fp32 with n numbers or a single one for
     all channels: the inputs of two sublayers that read the same rows through norms of
     their own."""
@@ -355,6 +359,10 @@ def add_norm2(x, a=None, b=None, rows=None, vec=None, eps: float = 0.0, w1=None,
                 y = t[:R].float() if y is None else y + t[:R].float()
         if vec is not None:
             y = vec if y is None else y + vec
+        if routed is not None:
+            ry, rw = routed
+            t = (ry[:R * rw.shape[1]].float().view(R, rw.shape[1], n) * rw[:R, :, None]).sum(1)
+            y = t if y is None else y + t
         if y is not None:
             x += y
         for w, o in ((w1, out1), (w2, out2)):
@@ -375,23 +383,33 @@ def add_norm2(x, a=None, b=None, rows=None, vec=None, eps: float = 0.0, w1=None,
         assert rows.dtype == torch.float32 and rows.is_contiguous() and rows.shape == x.shape
     if vec is not None:
         _vec(vec, n, "vec")
+    cy = cw = None
+    ldcy = top = 0
+    if routed is not None:
+        cy, cw = routed
+        top = cw.shape[1]
+        _rows2d(cy, "routed y")
+        assert cy.shape[1] == n and cy.shape[0] >= R * top and (a is None or cy.dtype == a.dtype)
+        assert cw.dtype == torch.float32 and cw.is_contiguous() and cw.shape[0] >= R
+        ldcy = cy.stride(0)
     ld1 = ld2 = 0
     for w, o, nm in ((w1, out1, "w1"), (w2, out2, "w2")):
         if w is not None:
             assert w.dtype == torch.float32 and w.is_contiguous() and w.numel() in (1, n), nm
             _rows2d(o, "out")
             assert o.shape[1] == n and o.shape[0] >= R and o.dtype == out1.dtype
-            assert a is None or o.dtype == a.dtype
+            assert (a is None or o.dtype == a.dtype) and (cy is None or o.dtype == cy.dtype)
     if out1 is not None:
         ld1 = out1.stride(0)
     if out2 is not None:
         ld2 = out2.stride(0)
-    act = a if a is not None else out1
+    act = a if a is not None else cy if cy is not None else out1
     _chk(lib().p2p_sm_add_norm2(x.data_ptr(), _lib.ptr(a), lda, _lib.ptr(b), ldb, _lib.ptr(rows),
                                 _lib.ptr(vec), R, n, eps, _lib.ptr(w1),
                                 1 if w1 is not None and w1.numel() > 1 else 0, _lib.ptr(out1), ld1,
                                 _lib.ptr(w2), 1 if w2 is not None and w2.numel() > 1 else 0,
-                                _lib.ptr(out2), ld2, _f32(act) if act is not None else 1, _st(x)),
+                                _lib.ptr(out2), ld2, _lib.ptr(cy), ldcy, _lib.ptr(cw), top,
+                                _f32(act) if act is not None else 1, _st(x)),
          "add_norm2")
     return x
 
@@ -887,6 +905,43 @@ def rope_rows(src, heads: int, src_hs: int, inv_freq, pos, dst, dst_hs: int, out
     return dst
 
 
+def latent_prep(proj, nq: int, nc: int, nr: int, qw, cw, inv_freq, pos, cache_rows, pool, eps: float,
+                cq_out):
+    """Input pass of latent attention with low-rank queries.  proj = [query latent (nq) |
+    key/value latent (nc) | key part (nr)] per row: both latents are RMS-normalised by
+    themselves and weighted (qw [nq], cw [nc]); the pairs (2i, 2i+1), i < len(inv_freq), of the
+    key part are turned by pos * inv_freq[i] (its other channels pass unchanged).  The query
+    latent goes to cq_out [R, nq], the key/value latent and the key part to the rows
+    ``cache_rows`` of the paged pool ([tokens, nc + nr]).  Norms, angles, rotation: fp32."""
+    R = cq_out.shape[0]
+    nrot = inv_freq.numel()
+    if not proj.is_cuda:
+        rows = cache_rows[:R].long()
+        cq_out[:R] = (_rms(proj[:R, :nq].float(), eps) * qw).to(cq_out.dtype)
+        pool[rows, :nc] = (_rms(proj[:R, nq:nq + nc].float(), eps) * cw).to(pool.dtype)
+        k = proj[:R, nq + nc:nq + nc + nr].float().clone()
+        ang = pos[:R].float()[:, None] * inv_freq[None, :]
+        c, sn = torch.cos(ang), torch.sin(ang)
+        a, b = k[:, 0:2 * nrot:2].clone(), k[:, 1:2 * nrot:2].clone()
+        k[:, 0:2 * nrot:2] = a * c - b * sn
+        k[:, 1:2 * nrot:2] = b * c + a * sn
+        pool[rows, nc:] = k.to(pool.dtype)
+        return cq_out
+    _rows2d(proj, "proj")
+    _rows2d(cq_out, "cq_out")
+    assert proj.shape[1] >= nq + nc + nr and cq_out.shape[1] == nq and cq_out.dtype == proj.dtype
+    assert pool.dim() == 2 and pool.is_contiguous() and pool.shape[1] == nc + nr and pool.dtype == proj.dtype
+    _vec(qw, nq, "qw")
+    _vec(cw, nc, "cw")
+    assert inv_freq.dtype == torch.float32 and inv_freq.is_contiguous() and 2 * nrot <= nr
+    assert pos.dtype == torch.int32 and cache_rows.dtype == torch.int32
+    _chk(lib().p2p_sm_latent_prep(proj.data_ptr(), proj.stride(0), nq, nc, nr, qw.data_ptr(),
+                                  cw.data_ptr(), inv_freq.data_ptr(), nrot, pos.data_ptr(),
+                                  cache_rows.data_ptr(), pool.data_ptr(), eps, cq_out.data_ptr(),
+                                  cq_out.stride(0), R, _f32(proj), _st(proj)), "latent_prep")
+    return cq_out
+
+
 def qtemp_kv_store(proj, nq: int, nkv: int, coef: float, every: int, pos, cache_rows, pool, q_out):
     """Prepares unrotated attention inputs from one projection buffer proj = [q (nq) | k and v
     (nkv)]: q goes to q_out multiplied by the query temperature of its position p,
@@ -1274,7 +1329,8 @@ ROUTE_SCORES = {"sigmoid": 0, "softmax": 1, "top_softmax": 2}
 
 
 def group_route(h, wr, top: int, groups: int, keep: int, ids, wts, cnt, rows,
-                score: str = "sigmoid", corr=None, group_score: str = "top2", bias=None):
+                score: str = "sigmoid", corr=None, group_score: str = "top2", bias=None,
+                cleared: bool = False):
     """Router with group-limited choice.  z = h wr^T (+ bias, fp32 [E]) in fp32 (wr fp32
     [E, W]); the scores are s = sigmoid(z) or (``score`` "softmax") softmax(z) over all E, or
     (``score`` "top_softmax") s = z for the choice and the weights are the softmax over the
@@ -1284,7 +1340,8 @@ def group_route(h, wr, top: int, groups: int, keep: int, ids, wts, cnt, rows,
     "top2") or by its best c ("max"), experts outside the ``keep`` best blocks are struck out;
     the ``top`` largest c among the rest win (ties: the lower index), their weights are their s.
     ids int32 / wts fp32 [R, top]; cnt int32 [E] and rows int32 [E, R*top] list per expert the
-    slots (row * top + k) routed to it (cnt is cleared here)."""
+    slots (row * top + k) routed to it (cnt is cleared here, unless the caller says it has
+    ``cleared`` it: a model clears the counts of all its layers with one fill per step)."""
     R = h.shape[0]
     E = wr.shape[0]
     per = E // groups
@@ -1303,7 +1360,7 @@ def group_route(h, wr, top: int, groups: int, keep: int, ids, wts, cnt, rows,
         i = masked.topk(top, dim=-1).indices
         ids[:R] = i.to(torch.int32)
         wts[:R] = s.gather(1, i) if score != "top_softmax" else torch.softmax(s.gather(1, i), -1)
-        cnt.zero_()
+        cnt.zero_()   # (the rendering fills the lists from scratch either way)
         for slot, e in enumerate(i.reshape(-1).tolist()):
             rows[e, int(cnt[e])] = slot
             cnt[e] += 1
@@ -1322,7 +1379,8 @@ def group_route(h, wr, top: int, groups: int, keep: int, ids, wts, cnt, rows,
     assert cnt.dtype == torch.int32 and cnt.numel() == E
     assert rows.dtype == torch.int32 and rows.is_contiguous() and rows.shape[0] == E \
         and rows.shape[1] >= R * top
-    cnt.zero_()
+    if not cleared:
+        cnt.zero_()
     _chk(lib().p2p_sm_group_route(h.data_ptr(), h.stride(0), wr.data_ptr(), R, h.shape[1], E, top,
                                   groups, keep, ROUTE_SCORES[score], _lib.ptr(corr),
                                   1 if group_score == "max" else 0, ids.data_ptr(),

@@ -35,7 +35,10 @@ def test_embed_scale_add_norm2(dt, wide):
     a, b = (torch.randn(R, W + 8, generator=g).to(dt)[:, 8:] for _ in range(2))
     rows, vec = torch.randn(R, W, generator=g), torch.randn(W, generator=g)
     one, two, per = torch.tensor([1.25]), torch.tensor([0.75]), 1 + 0.1 * torch.randn(W, generator=g)
-    cases = [dict(a=a), dict(a=a, b=b), dict(rows=rows, vec=vec), dict(a=a, b=b, rows=rows, vec=vec), dict(vec=vec), {}]
+    top = 3
+    ry, rw = torch.randn(R * top + 2, W, generator=g).to(dt), torch.rand(R, top, generator=g)
+    cases = [dict(a=a), dict(a=a, b=b), dict(rows=rows, vec=vec), dict(a=a, b=b, rows=rows, vec=vec), dict(vec=vec), {},
+             dict(a=a, routed=(ry, rw)), dict(routed=(ry, rw), rows=rows)]
     for kw in cases:
         for w1, w2 in ((None, None), (one, None), (one, two), (per, two), (per, per)):
             outs = []
@@ -43,7 +46,7 @@ def test_embed_scale_add_norm2(dt, wide):
                 x = x1.clone().to(dev)
                 h1 = torch.zeros(R, W, dtype=dt, device=dev) if w1 is not None else None
                 h2 = torch.zeros(R, W, dtype=dt, device=dev) if w2 is not None else None
-                args = {k: v.to(dev) for k, v in kw.items()}
+                args = {k: tuple(t.to(dev) for t in v) if isinstance(v, tuple) else v.to(dev) for k, v in kw.items()}
                 sm.add_norm2(x, eps=1e-5, w1=None if w1 is None else w1.to(dev), out1=h1,
                              w2=None if w2 is None else w2.to(dev), out2=h2, **args)
                 outs.append((x.cpu(), h1, h2))
@@ -84,6 +87,21 @@ def test_rope_rows_qtemp_gate_softcap(dt):
         sm.qtemp_kv_store(proj.to(DEV), nq, nkv, coef, every, pos2.to(DEV), rows.to(DEV), pb, qb)
         torch.testing.assert_close(qb.cpu().float(), qa.float(), **_tol(dt))
         torch.testing.assert_close(pb.cpu().float(), pa.float(), rtol=0, atol=0)
+    # both latents normed, the key part rotated (two of its channels pass unchanged), in one pass
+    nq, nc, nr = 37, 70, 2 * nrot + 2
+    proj = torch.randn(R, nq + nc + nr + 3, generator=g).to(dt)
+    qw, cw = 1 + 0.1 * torch.randn(nq, generator=g), 1 + 0.1 * torch.randn(nc, generator=g)
+    ca, cb = torch.empty(R, nq, dtype=dt), torch.empty(R, nq, dtype=dt, device=DEV)
+    pa, pb = torch.zeros(40, nc + nr, dtype=dt), torch.zeros(40, nc + nr, dtype=dt, device=DEV)
+    sm.latent_prep(proj, nq, nc, nr, qw, cw, inv, pos, rows, pa, 1e-5, ca)
+    sm.latent_prep(proj.to(DEV), nq, nc, nr, *_d(qw, cw, inv, pos, rows), pb, 1e-5, cb)
+    torch.testing.assert_close(cb.cpu().float(), ca.float(), **_tol(dt))
+    torch.testing.assert_close(pb.cpu().float(), pa.float(), **_tol(dt))
+    ref = sm.rmsnorm(proj[:, nq:nq + nc], cw, 1e-5, torch.empty(R, nc, dtype=dt))
+    torch.testing.assert_close(pa[rows.long(), :nc].float(), ref.float(), **_tol(dt))
+    kr = sm.rope_rows(proj[:, nq + nc:], 1, 0, inv, pos, torch.zeros(R, nr, dtype=dt), 0)
+    torch.testing.assert_close(pa[rows.long(), nc:nc + 2 * nrot].float(), kr[:, :2 * nrot].float(), **_tol(dt))
+    assert (pa[rows.long(), nc + 2 * nrot:] == proj[:, nq + nc + 2 * nrot:nq + nc + nr]).all()
     # one gate per head
     Vd = 20
     o, gt = torch.randn(H, R, Vd, generator=g).to(dt), torch.randn(R, H + 3, generator=g).to(dt)

@@ -119,6 +119,7 @@ __global__ void rope_rows_k(const T* __restrict__ src, int lds_, int heads, int 
 // weighted; the query latent goes to its own buffer, the key/value latent and the rotated part
 // to the token's row of the paged pool ([nc | nr]).  Wavefront 0 takes the query latent,
 // wavefront 1 the key/value latent, wavefront 2 the rotation.
+#define LP_NV 24   // values a lane keeps in registers: latents of up to 1536 numbers are read once
 template <typename T>
 __global__ void __launch_bounds__(192)
 latent_prep_k(const T* __restrict__ proj, int ldp, int nq, int nc, int nr,
@@ -135,6 +136,25 @@ latent_prep_k(const T* __restrict__ proj, int ldp, int nq, int nc, int nr,
     const float* w = wave ? cw : qw;
     T* dst = wave ? crow : cq + (size_t)r * ldq;
     float ss = 0.0f;
+    if (n <= 64 * LP_NV) {
+      // the latent and its weights are read once, all loads in flight together
+      float v[LP_NV], wv[LP_NV];
+#pragma unroll
+      for (int k = 0; k < LP_NV; k++) {
+        int i = lane + 64 * k;
+        v[k] = i < n ? ldf(src, i) : 0.0f;
+        wv[k] = i < n ? w[i] : 0.0f;
+        ss += v[k] * v[k];
+      }
+      ss = wave_sum(ss);
+      const float rs = 1.0f / sqrtf(ss / (float)n + eps);
+#pragma unroll
+      for (int k = 0; k < LP_NV; k++) {
+        int i = lane + 64 * k;
+        if (i < n) stf(dst, i, v[k] * rs * wv[k]);
+      }
+      return;
+    }
     for (int i = lane; i < n; i += 64) {
       float v = ldf(src, i);
       ss += v * v;

@@ -199,7 +199,7 @@ __global__ void add_norm_k(float* __restrict__ x, const T* __restrict__ a, int l
 // updated row, h_i = x / sqrt(mean(x^2) + eps) * w_i, where w_i is a vector (ws_i = 1) or one
 // number for all channels (ws_i = 0): two sublayers that read the same row through norms of
 // their own get their inputs from one pass over it.
-template <typename T>
+template <typename T, int NR>   // NR: values a thread keeps (rows of up to 256 * NR numbers are read once)
 __global__ void add_norm2_k(float* __restrict__ x, const T* __restrict__ a, int lda,
                             const T* __restrict__ b, int ldb, const float* __restrict__ rows,
                             const float* __restrict__ vec, int n, float eps,
@@ -218,58 +218,62 @@ __global__ void add_norm2_k(float* __restrict__ x, const T* __restrict__ a, int 
   const bool adds = ar || br || er || vec || cyr;
   // weights that are one number are read before the reduction
   const float g1 = (w1 && !ws1) ? w1[0] : 1.0f, g2 = (w2 && !ws2) ? w2[0] : 1.0f;
-  if (n <= NV * (int)blockDim.x) {
+  if (n <= NR * (int)blockDim.x) {
     // every load goes out before the first store; each addend's loads form one batch (the
     // tests for the optional addends stay outside the unrolled loops)
-    float xv[NV], yv[NV];
+    float xv[NR], yv[NR];
     float s2 = 0.0f;
 #pragma unroll
-    for (int k = 0; k < NV; k++) {
+    for (int k = 0; k < NR; k++) {
       int i = threadIdx.x + k * blockDim.x;
       xv[k] = xr[i < n ? i : 0];
       yv[k] = 0.0f;
     }
     if (ar) {
 #pragma unroll
-      for (int k = 0; k < NV; k++) {
+      for (int k = 0; k < NR; k++) {
         int i = threadIdx.x + k * blockDim.x;
         yv[k] = ldf(ar, i < n ? i : 0);
       }
     }
     if (br) {
 #pragma unroll
-      for (int k = 0; k < NV; k++) {
+      for (int k = 0; k < NR; k++) {
         int i = threadIdx.x + k * blockDim.x;
         yv[k] += ldf(br, i < n ? i : 0);
       }
     }
     if (er) {
 #pragma unroll
-      for (int k = 0; k < NV; k++) {
+      for (int k = 0; k < NR; k++) {
         int i = threadIdx.x + k * blockDim.x;
         yv[k] += er[i < n ? i : 0];
       }
     }
     if (vec) {
 #pragma unroll
-      for (int k = 0; k < NV; k++) {
+      for (int k = 0; k < NR; k++) {
         int i = threadIdx.x + k * blockDim.x;
         yv[k] += vec[i < n ? i : 0];
       }
     }
     if (cyr) {
-      for (int t = 0; t < top; t++) {
-        const float wt = cwr[t];
-        const T* yr = cyr + (size_t)t * ldcy;
+      // two experts at a time, so that a choice of two is one batch of loads
+      for (int t = 0; t < top; t += 2) {
+        const bool two = t + 1 < top;
+        const float wa = cwr[t], wb = two ? cwr[t + 1] : 0.0f;
+        const T* ya = cyr + (size_t)t * ldcy;
+        const T* yb = cyr + (size_t)(two ? t + 1 : t) * ldcy;
 #pragma unroll
-        for (int k = 0; k < NV; k++) {
+        for (int k = 0; k < NR; k++) {
           int i = threadIdx.x + k * blockDim.x;
-          yv[k] += wt * ldf(yr, i < n ? i : 0);
+          int ic = i < n ? i : 0;
+          yv[k] += wa * ldf(ya, ic) + wb * ldf(yb, ic);
         }
       }
     }
 #pragma unroll
-    for (int k = 0; k < NV; k++) {
+    for (int k = 0; k < NR; k++) {
       int i = threadIdx.x + k * blockDim.x;
       xv[k] = i < n ? xv[k] + yv[k] : 0.0f;
       if (adds && i < n) xr[i] = xv[k];
@@ -279,7 +283,7 @@ __global__ void add_norm2_k(float* __restrict__ x, const T* __restrict__ a, int 
     s2 = block_sum(s2, red);
     float r2 = 1.0f / sqrtf(s2 / (float)n + eps);
 #pragma unroll
-    for (int k = 0; k < NV; k++) {
+    for (int k = 0; k < NR; k++) {
       int i = threadIdx.x + k * blockDim.x;
       if (i < n) {
         float v = xv[k] * r2;
@@ -448,10 +452,16 @@ int p2p_sm_add_norm2(float* x, const void* a, int lda, const void* b, int ldb, c
   if (R <= 0) return 0;
   if ((w1 && !h1) || (w2 && (!h2 || !w1)) || (b && !a) || (cy && (!cw || top < 1)))
     return (int)hipErrorInvalidValue;
-  SM_DISPATCH_T(f32, hipLaunchKernelGGL(add_norm2_k<T>, dim3(R), dim3(256), 0, st, x, (const T*)a,
-                                         lda, (const T*)b, ldb, rows, vec, n, eps, w1, ws1,
-                                         (T*)h1, ld1, w2, ws2, (T*)h2, ld2, (const T*)cy, ldcy,
-                                         cw, top));
+#define AN2(NR)                                                                                 \
+  SM_DISPATCH_T(f32, hipLaunchKernelGGL((add_norm2_k<T, NR>), dim3(R), dim3(256), 0, st, x,     \
+                                         (const T*)a, lda, (const T*)b, ldb, rows, vec, n, eps,  \
+                                         w1, ws1, (T*)h1, ld1, w2, ws2, (T*)h2, ld2,             \
+                                         (const T*)cy, ldcy, cw, top))
+  // the smallest instance whose registers hold the row: no loads of padding, less code to fetch
+  if (n <= 256 * 4) AN2(4);
+  else if (n <= 256 * 8) AN2(8);
+  else AN2(16);
+#undef AN2
   return (int)hipGetLastError();
 }
 

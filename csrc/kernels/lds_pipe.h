@@ -5,9 +5,9 @@
 // ds_read.  Written with the builtins, the compiler cannot tell which LDS bytes a pending
 // DMA writes, and with DMA events pending it gives up on counting: it puts s_waitcnt
 // vmcnt(0) before every ds_read (and every use of a register loaded after a DMA), so each
-// k-tile waited for ALL loads in flight and the pipeline drained at every step (round-6
-// disassembly of both kernels).  Issued as asm, these loads and reads are invisible to the
-// compiler's wait insertion: the kernels' own counted waits are the only ones.
+// k-tile waited for ALL loads in flight and the pipeline drained at every step.  Issued as
+// asm, these loads and reads are invisible to the compiler's wait insertion: the kernels' own
+// counted waits are the only ones.
 //
 // Rules for a kernel using them:
 //  * every load the k loop depends on is issued here (dma_lds / gload_nt) and waited for by

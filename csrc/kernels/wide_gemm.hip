@@ -84,7 +84,7 @@ __device__ __forceinline__ void wait_vmcnt() {
 // (global_load_lds), and the compiler cannot tell which ring slot a pending DMA writes: it
 // put an s_waitcnt vmcnt(0) before every ds_read of the ring, so each chunk's compute waited
 // for ALL loads in flight (the next D chunks' weights and activations too) and the pipeline
-// drained at every chunk (r6 disassembly; gate_up 16 x 2.8 us per chunk on the ring path).
+// drained at every chunk (gate_up: 16 x 2.8 us per chunk on the ring path).
 // The kernel's own counted vmcnt wait + barrier already makes chunk t's slot complete, so
 // the reads go out as asm (the compiler inserts no wait for them) and lds_wait holds their
 // results until they land.

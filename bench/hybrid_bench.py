@@ -99,14 +99,14 @@ def tarunex_config(width: int):
            "router": {"experts": 8, "top": 2}}
     ba = {"type": "attention",
           "mixer": {"heads": nh, "kv_heads": max(1, nh // 4), "dim": hd, "vdim": hd, "scale": hd ** -0.5,
-                    "softcap": 30.0, "q_temp": {"coef": 0.1, "every": 512}}, "mlp": moe}
+                    "softcap": 50.0, "q_temp": {"coef": 0.1, "every": 512}}, "mlp": moe}
     la = {"type": "latent_attention",
           "mixer": {"heads": nh, "dim": hd, "rot_dim": 64, "vdim": hd, "kv_rank": 448, "q_rank": width // 2,
                     "rot": {"base": 10000.0, "dims": 64}, "scale": (hd + 64) ** -0.5}, "mlp": moe}
     layers = [ba, ba, ba, la, ba, ba, la, ba, ba, la]
     return HybridConfig.from_dict(
         {"architecture": "Tarunex", "width": width, "vocab": 32000, "norm": {"eps": 1e-5},
-         "embedding": {"scale": width ** 0.5}, "logit_scale": 0.25, "logit_softcap": 30.0,
+         "embedding": {"scale": width ** 0.5}, "logit_scale": 0.5, "logit_softcap": 50.0,
          "loop": {"start": 2, "stop": 8, "times": 2}, "layers": layers}, name="tarunex-w%d" % width)
 
 

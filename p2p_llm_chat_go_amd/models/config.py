@@ -124,7 +124,7 @@ def _hybrid_presets() -> dict:
     smoe = {"kind": "moe", "expert": {"ff": 128}, "shared": {"ff": 256},
             "router": {"experts": 6, "identity": 2, "top": 2, "groups": {"count": 4, "keep": 2}}}
     ba = {"type": "attention",
-          "mixer": {"heads": 8, "kv_heads": 2, "dim": 32, "vdim": 32, "scale": 32 ** -0.5, "softcap": 30.0,
+          "mixer": {"heads": 8, "kv_heads": 2, "dim": 32, "vdim": 32, "scale": 32 ** -0.5, "softcap": 20.0,
                     "q_temp": {"coef": 0.1, "every": 128}}}
     rl = {"type": "latent_attention",
           "mixer": {"heads": 4, "dim": 32, "rot_dim": 16, "vdim": 32, "kv_rank": 64, "q_rank": 96,
@@ -145,7 +145,7 @@ def _hybrid_presets() -> dict:
          "eos_token_id": [2]}, name="tiny-futetar"),
         "tiny-tarunex": HybridConfig.from_dict(
         {"architecture": "Tarunex", "width": 256, "vocab": 512, "norm": {"eps": 1e-5},
-         "embedding": {"scale": 16.0}, "logit_scale": 0.5, "logit_softcap": 30.0,
+         "embedding": {"scale": 16.0}, "logit_scale": 0.5, "logit_softcap": 25.0,
          "loop": {"start": 1, "stop": 3, "times": 2},
          "layers": [dict(ba, mlp=tmoe), dict(rl, mlp=tmoe), dict(ba, mlp=tmoe), dict(rl, mlp=None)],
          "eos_token_id": [2]}, name="tiny-tarunex")}

@@ -80,7 +80,7 @@ def test_rope_rows_qtemp_gate_softcap(dt):
     nq, nkv = 35, 27
     proj = torch.randn(R, nq + nkv + 6, generator=g).to(dt)
     pos2 = torch.tensor([0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 14, 15, 16, 63, 64, 1000, 4095], dtype=torch.int32)
-    for coef, every in ((0.7, 4), (0.0, 1), (2.0, 1), (0.3, 64)):
+    for coef, every in ((0.7, 4), (0.0, 1), (2.0, 1), (0.25, 32)):
         qa, qb = torch.empty(R, nq, dtype=dt), torch.empty(R, nq, dtype=dt, device=DEV)
         pa, pb = torch.zeros(40, nkv, dtype=dt), torch.zeros(40, nkv, dtype=dt, device=DEV)
         sm.qtemp_kv_store(proj, nq, nkv, coef, every, pos2, rows, pa, qa)
@@ -202,7 +202,7 @@ def test_latent_attn_without_sink(dt, H, rank, win):
 
 
 @pytest.mark.parametrize("dt", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("E,top,W,Fd", [(12, 4, 72, 48), (8, 2, 64, 64), (6, 6, 50, 33), (70, 5, 96, 32), (2, 1, 40, 16)])
+@pytest.mark.parametrize("E,top,W,Fd", [(10, 4, 72, 48), (8, 2, 64, 64), (6, 6, 50, 33), (70, 5, 96, 32), (2, 1, 40, 16)])
 @pytest.mark.parametrize("R", [45, 300])     # few slots per expert / the large prompt tile
 def test_router_bias_and_silu_experts(dt, E, top, W, Fd, R):
     g = torch.Generator().manual_seed(5)

@@ -1,10 +1,13 @@
 """Sequence-mixer ops: recurrent state layers (generalized delta rule, Mamba-2, gated delta
-rule, HGRN2, the mLSTM's matrix memory), latent attention and grouped-query attention with an
-optional sliding window and softmax sink (query/key norm over the row or per head, rotary
-positions on adjacent or half-split channel pairs and the cache write in one pass), a
-group-limited expert router (sigmoid or softmax scores, optional score correction) with
-grouped expert products and identity experts, learned positions, and the norms, residual
-passes and pointwise steps around them.
+rule, HGRN2, the mLSTM's matrix memory), latent attention (optionally with a rotated key part
+in the cached row and without a sink) and grouped-query attention with an optional sliding
+window and softmax sink (query/key norm over the row or per head, rotary positions on adjacent
+or half-split channel pairs and the cache write in one pass; or unrotated with a query
+temperature, capped scores, a logarithmic distance penalty and a gate per head), a
+group-limited expert router (sigmoid or softmax scores, optional score correction and bias,
+softmax over the chosen logits) with grouped expert products and identity experts, learned
+positions, and the norms, residual passes (one with two normed outputs and the routed experts'
+weighted sum) and pointwise steps around them.
 
 GPU tensors always run the gfx950 kernels of ``csrc/seqmix`` (``libp2p_seqmix.so``, built on
 first use when missing); CPU tensors run the PyTorch rendering of the same math, which is

@@ -180,7 +180,7 @@ VARIANTS = {
     "odd": ([layer(BA, {"kind": "moe", "expert": {"ff": 10}, "router": {"experts": 3, "top": 3}},
                    heads=5, kv_heads=5, dim=6, vdim=10, scale=0.05, softcap=2.0),
              layer(LA, {"kind": "dense", "ff": 50}, heads=5, dim=6, rot_dim=6, vdim=4, kv_rank=13, q_rank=9,
-                   rot={"base": 40000.0, "dims": 6}),
+                   rot={"base": 40000.0, "dims": 4}),      # the last pair of the key part is not rotated
              layer(BA, None, heads=3, kv_heads=1, dim=10, vdim=6, q_temp={"coef": 1.5, "every": 7})],
             (1, 3, 2)),
     # wide heads and latents, value size above key size, the stretch of passes at the end
